@@ -26,9 +26,14 @@ extern "C" {
 typedef struct ihipStream_t* umb_stream_t;   /* == hipStream_t */
 
 enum { UMB_SEQ_F16 = 0, UMB_SEQ_BF16 = 1, UMB_SEQ_F32 = 2 };
-enum { UMB_MIX_POOLED_WINDOW = 0, UMB_MIX_GLA = 1, UMB_MIX_LATENT = 2 };
+enum { UMB_MIX_POOLED_WINDOW = 0, UMB_MIX_GLA = 1, UMB_MIX_LATENT = 2, UMB_MIX_MINGRU = 3, UMB_MIX_ATTN_SSD = 4 };
 /* feed-forward kinds: gated SiLU (W_down (silu(W_gate h) * W_up h)), PolyNorm (W_down polynorm(W_up h)), routed experts */
 enum { UMB_FF_GATED = 0, UMB_FF_POLYNORM = 1, UMB_FF_MOE = 2 };
+/* activation of a feed-forward / expert: silu(W_gate h) * (W_up h) over stacked [gate; up], or relu(W_up h)^2 (no gate) */
+enum { UMB_ACT_SILU_GATED = 0, UMB_ACT_RELU2 = 1 };
+/* routing of experts: sigmoid scores that multiply the expert's input; or softmax scores, chosen with a correction added,
+ * renormalised over the chosen ones, that multiply the expert's output */
+enum { UMB_ROUTE_SIGMOID_IN = 0, UMB_ROUTE_SOFTMAX_OUT = 1 };
 
 /* W [N][K] row-major (as stored: out x in), optional bias [N]; applied as W x + b */
 typedef struct UmbSeqLinear { const void* w; const void* bias; int32_t N, K; } UmbSeqLinear;
@@ -37,7 +42,7 @@ typedef struct UmbSeqLinear { const void* w; const void* bias; int32_t N, K; } U
 
 /* out[T][N] = x[T][K] . W^T + bias, fp32 accumulation in a fixed order that depends on (N, K) only.
  * epi 0: out fp32; epi 1: out in `dtype`; epi 2: W stacks [gate; up] (N = 2 N'), out[T][N'] in `dtype` =
- * silu(gate) * up.  x and W in `dtype`. */
+ * silu(gate) * up; epi 4: out in `dtype` = relu(acc)^2.  x and W in `dtype`. */
 int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, int dtype,
                    umb_stream_t stream);
 
@@ -103,7 +108,7 @@ int umb_moe_route(int* sel, float* wt, const float* logits, int T, int E, int to
  * (max_tiles >= ceil(T top / tile_rows) + E; unused entries get rows = 0). */
 int umb_moe_plan(int* pos_of, int* tiles, const int* sel, int T, int E, int top, int max_tiles, int tile_rows,
                  umb_stream_t stream);
-/* xs[pos_of[t top + k]] = wt[t][k] * h[t]  (the weight multiplies the expert's INPUT); h, xs in `dtype` */
+/* xs[pos_of[t top + k]] = wt[t][k] * h[t]  (the weight multiplies the expert's INPUT; wt null: 1); h, xs in `dtype` */
 int umb_moe_scatter(void* xs, const void* h, const float* wt, const int* pos_of, int T, int W, int top, int dtype,
                     umb_stream_t stream);
 /* y[t] = (add ? y[t] : 0) + sum_k ye[pos_of[t top + k]]  (k ascending) */
@@ -177,6 +182,81 @@ int umb_lat_attend_tiled(void* out, const float* qa, const UmbPagedKV* kv, const
                          const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int max_len, int H, int kv_rank,
                          int rot_dim, int window, float scale, int dtype, umb_stream_t stream);
 
+/* ---- several residual streams ("hyper-connections").  The residual is S copies per token, x fp32 [T][S][W].  A sublayer
+ * reads u = sum_s in[s] x_s through an RMS norm whose weight is stored around `offset` (h = u / rms(u) * (offset + w));
+ * its output y is written back to all streams at once from the old ones: x_t <- sum_s mix[s][t] x_s + m out[t] y.
+ * in / out / mix are fp32 and may be null (all ones / all ones / identity); S = 1 with nulls is the plain x + m y.
+ * embed: every stream <- embed[token] * scale, h <- first read.  seam: write of the sublayer behind, read of the one ahead
+ * (in_next null and w_next null: no read).  read: rows gathered through `rows` (null: all), u_out (fp32 [R][W]) and / or
+ * h may be given; in null sums the streams. */
+int umb_hc_embed(float* x, void* h, const void* embed, const int* tokens, float scale, const float* in, const void* w,
+                 float offset, int T, int W, int V, int S, float eps, int dtype, umb_stream_t stream);
+int umb_hc_seam(float* x, void* h, const float* y, const float* mix, const float* out, float m, const float* in_next,
+                const void* w_next, float offset, int T, int W, int S, float eps, int dtype, umb_stream_t stream);
+int umb_hc_read(float* u_out, void* h, const float* x, const int* rows, const float* in, const void* w, float offset, int R,
+                int W, int S, float eps, int dtype, umb_stream_t stream);
+
+/* ---- minimal gated recurrence, element by element over `Wm` channels: with the projections zr / ur / gr (fp32, biases
+ * added, columns z_col / u_col / g_col of proj [T][ld]), z = sigmoid(zr), candidate = ur + 1/2 where ur >= 0, else
+ * sigmoid(ur); S_t = (1 - z) S_(t-1) + z candidate; out[t] = S_t * silu(gr) in `dtype`.  state fp32 [slots][Wm]; a
+ * sequence that starts at position 0 starts from S = 0 whatever its slot holds. */
+int umb_mingru_scan(void* out, float* state, const float* proj, int ld, int z_col, int u_col, int g_col, const int* seq_slot,
+                    const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int Wm, int dtype, umb_stream_t stream);
+
+/* ---- linear recurrence with a matrix state per head, general operand placement (umb_gla_scan is one case of it):
+ * S <- a_t S + k_t v_t^T, o_t = S^T (q_t * qscale); q and k rows [T][ldq / ldk] hold qk_heads groups of D (head h reads
+ * group h / (H / qk_heads)), v rows H heads of Dv; the decay is per key channel (alpha [T][H D], alpha_per_head 0) or one
+ * number per head (alpha [T][H], alpha_per_head 1).  state fp32 [slots][H][D][Dv]. */
+int umb_lin_scan(float* o, float* state, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                 const float* alpha, int alpha_per_head, int qk_heads, const int* seq_slot, const int* seq_row0,
+                 const int* seq_pos0, const int* seq_len, int B, int H, int D, int Dv, float qscale, umb_stream_t stream);
+
+/* ---- selective state space with a scalar decay per head (state-space duality).  proj fp32 [T][ld]; from column col0:
+ * [z (H Dv) | x (H Dv) | B (G N) | C (G N) | dt (H)].  prep: x, B, C through a causal convolution per channel (w [C][taps],
+ * last column the token's own, bias b, inputs of earlier steps from conv_state fp32 [slots][taps - 1][C], the input of
+ * position p in row p % (taps - 1)) and silu; dt = softplus(dt + dt_bias[h]); sx fp32 [T][lds] = [dt x | B | C | x],
+ * alpha [T][H] = exp(-exp(a_log[h]) dt).  conv_update, launched after prep, stores the step's last raw inputs.
+ * The recurrence itself is umb_lin_scan (k = B, v = dt x, q = C).
+ * gate: y = o + d_skip[h] x, times silu(z), unit RMS in `norm_groups` equal parts of the H Dv row, times w, times
+ * out_scale, in `dtype` at out[t ldo + ...]. */
+int umb_ssd_prep(float* sx, int lds, float* alpha, const float* proj, int ld, int col0, const void* conv_w, const void* conv_b,
+                 const float* conv_state, const float* dt_bias, const float* a_log, const int* pos, const int* slot, int T, int H,
+                 int Dv, int G, int N, int taps, int dtype, umb_stream_t stream);
+int umb_ssd_conv_update(float* conv_state, const float* proj, int ld, int col0, const int* seq_slot, const int* seq_row0,
+                        const int* seq_pos0, const int* seq_len, int B, int C, int taps, umb_stream_t stream);
+int umb_ssd_gate(void* out, int ldo, const float* o, const float* sx, int lds, int x_col, const float* proj, int ld, int z_col,
+                 const float* d_skip, const void* w, int T, int H, int Dv, int norm_groups, float eps, float out_scale, int dtype,
+                 umb_stream_t stream);
+
+/* ---- causal softmax attention with a bias by distance over a paged store (UmbPagedKV: k [pages][G][page][D],
+ * v [pages][G][page][E] in `dtype`; kp / vp unused).  proj fp32 [T][ld] = [q (H D) | k (G D) | v (G E) | gate (H)].
+ * prep: q <- unit_rms(q) * w_q * (1 + temp_coef ln(floor((pos + 1) / temp_every) + 1)), fp32 [T][H D] (w_q, w_k [D], shared by
+ * the heads; null: 1); cache K <- unit_rms(k) * w_k; cache V <- unit_rms(v) (no weight).
+ * attend: score(i, j, h) = q_i . k_j * scale + bias[h][min(i - j, n_dist - 1)] over j <= i with i - j < window (bias fp32
+ * [H][n_dist], null: none); softmax; out[t ldo + h E ..] = out_scale * sigmoid(gate[t][h]) * sum_j p_j v_j in `dtype`
+ * (gate_col < 0: no gate). */
+int umb_bsa_prep(float* q, const UmbPagedKV* kv, const float* proj, int ld, const void* w_q, const void* w_k, const int* pos,
+                 const int* slot, int T, int H, int G, int D, int E, float temp_coef, int temp_every, float eps, int dtype,
+                 umb_stream_t stream);
+int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
+                   const float* bias, int n_dist, const int* pos, const int* slot, int T, int H, int G, int D, int E, int window,
+                   float scale, float out_scale, int dtype, umb_stream_t stream);
+/* the same for steps that bring stretches of a sequence, on the matrix pipe (16-bit storage; umb_bsa_attend_tiled_ok says
+ * 1 / 0 whether the kernel covers a shape and dtype; it has no stream): workgroups own 16 consecutive positions */
+int umb_bsa_attend_tiled_ok(int H, int G, int D, int E, int dtype);
+int umb_bsa_attend_tiled(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
+                         const float* bias, int n_dist, const int* seq_slot, const int* seq_row0, const int* seq_pos0,
+                         const int* seq_len, int B, int max_len, int H, int G, int D, int E, int window, float scale,
+                         float out_scale, int dtype, umb_stream_t stream);
+
+/* ---- routed experts, softmax form: scores = softmax(logits) over all experts; the `top` largest of score + correction
+ * (correction fp32 [E], null: none; ties: the lower index) are chosen; wt = the chosen scores over (their sum + 1e-20). */
+int umb_moe_route_softmax(int* sel, float* wt, const float* logits, const float* correction, int T, int E, int top,
+                          umb_stream_t stream);
+/* y[t] = (add ? y[t] : 0) + sum_k wt[t top + k] * ye[pos_of[t top + k]]  (k ascending) */
+int umb_moe_combine_weighted(float* y, const float* ye, const float* wt, const int* pos_of, int T, int W, int top, int add,
+                             umb_stream_t stream);
+
 /* ------------------------------------------------------------------ the model */
 typedef struct UmbSeqLayer {
   int32_t kind, has_mlp;
@@ -212,6 +292,25 @@ typedef struct UmbSeqLayer {
   const void* e_gu;       /* [experts][2 expert_ff][W]: every expert's stacked [gate; up] */
   const void* e_down;     /* [experts][W][expert_ff] */
   UmbSeqLinear s_gu, s_down;   /* shared expert (s_gu.w null: none) */
+  /* act: UMB_ACT_* of the dense feed-forward, the experts and the shared expert (relu^2: gu / e_gu / s_gu hold the
+   * up-projection alone); route: UMB_ROUTE_*; correction fp32 [experts] (softmax routing, may be null) */
+  int32_t act_kind, route_kind;
+  const float* correction;
+  /* several residual streams (model.streams >= 1): read / write / mix weights of the two sublayers, fp32, null = trivial */
+  const float *hc1_in, *hc1_out, *hc1_mix, *hc2_in, *hc2_out, *hc2_mix;
+  /* minGRU (kind 3): proj = [z | x | g], each `dim` wide; state [slots][dim] fp32.
+   * attention beside a state-space layer (kind 4), both reading the same input: proj = [q | k | v | gate | z | x | B | C | dt];
+   * attention: heads / kv_heads / dim / vdim / scale / window, q_norm / k_norm [dim], dist_bias fp32 [heads][n_dist],
+   * query temperature; state space: s_heads x s_vdim, state size s_state, s_groups groups of B / C, s_taps convolution taps;
+   * the output projection reads [mix_scale_a * attention | mix_scale_b * state space] */
+  const void *q_norm, *k_norm;
+  const float* dist_bias;
+  int32_t n_dist, temp_every;
+  float temp_coef, mix_scale_a, mix_scale_b, pad3_;
+  int32_t s_heads, s_vdim, s_state, s_groups, s_norm_groups, s_taps;
+  const void *s_conv, *s_conv_b, *s_norm;
+  const float *s_dt_bias, *s_a_log, *s_d;
+  float* s_conv_state;        /* [slots][s_taps - 1][channels] fp32 */
 } UmbSeqLayer;
 
 typedef struct UmbSeqModel {
@@ -219,11 +318,16 @@ typedef struct UmbSeqModel {
   float eps, embed_scale;    /* embed_scale: the embedding row is multiplied by it (1: as stored) */
   const void* embed; const void* final_norm; UmbSeqLinear head;
   const UmbSeqLayer* layers;
+  /* streams >= 1: the residual is `streams` copies per token (ws.x is [Tmax][streams][W]), a sublayer is
+   * x <- mix x + resid_mult * out * f(norm(in . x)) with norm weights stored around norm_offset, and the model ends with
+   * the norm of the sum of the streams; 0: the single-stream forms above */
+  int32_t streams, pad_;
+  float resid_mult, norm_offset;
 } UmbSeqModel;
 
 /* activations of one step (caller-owned, sized for Tmax rows) */
 typedef struct UmbSeqWork {
-  float* x;        /* residual stream [Tmax][W] fp32 */
+  float* x;        /* residual stream [Tmax][W] fp32 ([Tmax][streams][W] with several streams) */
   void* h;         /* normed input of the current sublayer [Tmax][W] dtype */
   float* proj;     /* fused projection output [Tmax][max proj N] fp32 */
   float* aux;      /* q / alpha [Tmax][max heads*dim] fp32 */
@@ -249,7 +353,7 @@ typedef struct UmbSeqStep {
   const int32_t *tokens, *pos, *slot;                       /* [T] */
   const int32_t *seq_slot, *seq_row0, *seq_pos0, *seq_len;  /* [B] */
   const int32_t* logit_rows;                                /* [R] rows whose logits are wanted */
-  float* trace;                                             /* optional [L][T][W]: the residual stream after every layer */
+  float* trace;                                             /* optional [L][T][W]: the residual stream after every layer (the sum of the streams) */
 } UmbSeqStep;
 
 int umb_lat_attend_tiled_ok(int H, int kv_rank, int rot_dim, int dtype);

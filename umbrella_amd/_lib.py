@@ -225,13 +225,24 @@ class UmbSeqLayer(C.Structure):
                 ("uq", UmbSeqLinear), ("uk_t", C.c_void_p), ("uv", C.c_void_p), ("dq_norm", C.c_void_p),
                 ("dkv_norm", C.c_void_p), ("sink", C.c_void_p), ("canon1", C.c_void_p), ("canon2", C.c_void_p),
                 ("canon_state1", C.c_void_p), ("canon_state2", C.c_void_p), ("act", C.c_void_p), ("router", UmbSeqLinear),
-                ("e_gu", C.c_void_p), ("e_down", C.c_void_p), ("s_gu", UmbSeqLinear), ("s_down", UmbSeqLinear)]
+                ("e_gu", C.c_void_p), ("e_down", C.c_void_p), ("s_gu", UmbSeqLinear), ("s_down", UmbSeqLinear),
+                ("act_kind", C.c_int32), ("route_kind", C.c_int32), ("correction", C.c_void_p),
+                ("hc1_in", C.c_void_p), ("hc1_out", C.c_void_p), ("hc1_mix", C.c_void_p),
+                ("hc2_in", C.c_void_p), ("hc2_out", C.c_void_p), ("hc2_mix", C.c_void_p),
+                ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("dist_bias", C.c_void_p),
+                ("n_dist", C.c_int32), ("temp_every", C.c_int32),
+                ("temp_coef", C.c_float), ("mix_scale_a", C.c_float), ("mix_scale_b", C.c_float), ("pad3_", C.c_float),
+                ("s_heads", C.c_int32), ("s_vdim", C.c_int32), ("s_state", C.c_int32), ("s_groups", C.c_int32),
+                ("s_norm_groups", C.c_int32), ("s_taps", C.c_int32),
+                ("s_conv", C.c_void_p), ("s_conv_b", C.c_void_p), ("s_norm", C.c_void_p),
+                ("s_dt_bias", C.c_void_p), ("s_a_log", C.c_void_p), ("s_d", C.c_void_p), ("s_conv_state", C.c_void_p)]
 
 
 class UmbSeqModel(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("L", C.c_int32), ("W", C.c_int32), ("V", C.c_int32), ("groups", C.c_int32),
                 ("canon_taps", C.c_int32), ("eps", C.c_float), ("embed_scale", C.c_float), ("embed", C.c_void_p),
-                ("final_norm", C.c_void_p), ("head", UmbSeqLinear), ("layers", C.POINTER(UmbSeqLayer))]
+                ("final_norm", C.c_void_p), ("head", UmbSeqLinear), ("layers", C.POINTER(UmbSeqLayer)),
+                ("streams", C.c_int32), ("pad_", C.c_int32), ("resid_mult", C.c_float), ("norm_offset", C.c_float)]
 
 
 class UmbSeqWork(C.Structure):
@@ -280,12 +291,26 @@ SEQ_SIGNATURES = {
     "umb_pwa_pool": [_PKV, _P, _P, _P, _I, _I, _I, _I, _I, _I],
     "umb_pwa_attend": [_P, _P, _PKV, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I],
     "umb_pwa_attend_tiled": [_P, _P, _PKV, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I],
+    "umb_hc_embed": [_P, _P, _P, _P, _F, _P, _P, _F, _I, _I, _I, _I, _F, _I],
+    "umb_hc_seam": [_P, _P, _P, _P, _P, _F, _P, _P, _F, _I, _I, _I, _F, _I],
+    "umb_hc_read": [_P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _F, _I],
+    "umb_mingru_scan": [_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I],
+    "umb_lin_scan": [_P, _P, _P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _F],
+    "umb_ssd_prep": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
+    "umb_ssd_conv_update": [_P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
+    "umb_ssd_gate": [_P, _I, _P, _P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I],
+    "umb_bsa_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I],
+    "umb_bsa_attend": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _I],
+    "umb_bsa_attend_tiled": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I],
+    "umb_bsa_attend_tiled_ok": [_I, _I, _I, _I, _I],
+    "umb_moe_route_softmax": [_P, _P, _P, _P, _I, _I, _I],
+    "umb_moe_combine_weighted": [_P, _P, _P, _P, _I, _I, _I, _I],
     "umb_seq_forward": [C.POINTER(UmbSeqModel), C.POINTER(UmbSeqWork), C.POINTER(UmbSeqStep)],
     "umb_argmax_rows": [_P, _P, _I, _I],
     "umb_sample_rows": [_P, _P, _I, _I, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P],
     "umb_seq_version": [],
 }
-_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok", "umb_seq_resid_canon_step_ok"}          # predicates: no stream argument, the value is the answer
+_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok", "umb_seq_resid_canon_step_ok", "umb_bsa_attend_tiled_ok"}          # predicates: no stream argument, the value is the answer
 _seq_lib = None
 
 

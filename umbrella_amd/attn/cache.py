@@ -149,7 +149,11 @@ class PagedSeqCache:
       key/value latent and the rotated key part that all heads share;
     * gated-linear-attention layers keep one fp32 state ``[slots, H, D, Dv]`` each;
     * a convolution in front of a sublayer keeps its last ``taps - 1`` inputs, fp32 ``[slots, taps - 1, W]`` per sublayer
-      (the input at position p in row p % (taps - 1));
+      (the input at position p in row p % (taps - 1)); a mixer's own input convolution does the same over its own channels
+      (``mixer_convs``: ``(taps, channels)`` each);
+    * softmax-attention layers with separate values keep K ``[pages, G, page, D]`` and V ``[pages, G, page, E]`` and no
+      pooled entries (a ``kv_layers`` entry ``(G, D, 0, E)``);
+    * element-wise recurrences use the same state arrays with ``(1, 1, channels)``;
     * nothing is cleared when a slot or a page is handed out again: a sequence that starts at position 0 ignores what its
       slot holds, and no kernel reads a cache position its own sequence has not written.
 
@@ -157,7 +161,7 @@ class PagedSeqCache:
     """
 
     def __init__(self, kv_layers, state_layers, max_tokens: int, max_seqs: int, device, dtype, page: int = 64,
-                 latent_layers=(), conv_states: int = 0, conv_taps: int = 0, width: int = 0):
+                 latent_layers=(), conv_states: int = 0, conv_taps: int = 0, width: int = 0, mixer_convs=()):
         assert page >= 1 and max_tokens >= 1 and max_seqs >= 1
         self.page, self.max_seqs, self.device, self.dtype = int(page), int(max_seqs), device, dtype
         # every sequence may leave one page partly filled
@@ -165,18 +169,24 @@ class PagedSeqCache:
         self.max_pages = self.n_pages
         self.pages_dev = torch.zeros(max_seqs, self.max_pages, dtype=torch.int32, device=device)
         self.kv, self.state = [], []
-        for (G, D, pool) in kv_layers:
-            npb = (page + pool - 1) // pool
-            self.kv.append(dict(
-                k=torch.zeros(self.n_pages, G, page, D, dtype=dtype, device=device),
-                v=torch.zeros(self.n_pages, G, page, D, dtype=dtype, device=device),
-                kp=torch.zeros(self.n_pages, G, npb, D, dtype=torch.float32, device=device),
-                vp=torch.zeros(self.n_pages, G, npb, D, dtype=torch.float32, device=device), G=G, D=D, pool=pool))
+        for spec in kv_layers:
+            G, D, pool = spec[:3]
+            E = spec[3] if len(spec) > 3 else D                         # value size (pooled layers: the key size)
+            entry = dict(k=torch.zeros(self.n_pages, G, page, D, dtype=dtype, device=device),
+                         v=torch.zeros(self.n_pages, G, page, E, dtype=dtype, device=device), kp=None, vp=None, G=G, D=D, E=E,
+                         pool=pool)
+            if pool > 0:
+                npb = (page + pool - 1) // pool
+                entry["kp"] = torch.zeros(self.n_pages, G, npb, D, dtype=torch.float32, device=device)
+                entry["vp"] = torch.zeros(self.n_pages, G, npb, D, dtype=torch.float32, device=device)
+            self.kv.append(entry)
         for (H, D, Dv) in state_layers:
             self.state.append(torch.zeros(max_seqs, H, D, Dv, dtype=torch.float32, device=device))
         self.latent = [torch.zeros(self.n_pages, page, Dk, dtype=dtype, device=device) for Dk in latent_layers]
         self.conv = [torch.zeros(max_seqs, max(conv_taps - 1, 1), width, dtype=torch.float32, device=device)
                      for _ in range(conv_states)] if conv_taps > 0 else []
+        self.mixer_conv = [torch.zeros(max_seqs, max(taps - 1, 1), ch, dtype=torch.float32, device=device)
+                           for (taps, ch) in mixer_convs]
         self.clear()
 
     def clear(self):
@@ -263,6 +273,7 @@ class PagedSeqCache:
     def struct(self, layer: int) -> "_lib.UmbPagedKV":
         c = self.kv[layer]
         kv = _lib.UmbPagedKV()
-        kv.k, kv.v, kv.kp, kv.vp = c["k"].data_ptr(), c["v"].data_ptr(), c["kp"].data_ptr(), c["vp"].data_ptr()
+        kv.k, kv.v = c["k"].data_ptr(), c["v"].data_ptr()
+        kv.kp, kv.vp = (c["kp"].data_ptr(), c["vp"].data_ptr()) if c["kp"] is not None else (None, None)
         kv.pages, kv.max_pages, kv.page, kv.n_pages = self.pages_dev.data_ptr(), self.max_pages, self.page, self.n_pages
         return kv

@@ -89,6 +89,51 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int* __restrict__ sel, f
   }
 }
 
+// Softmax routing: scores = softmax(logits) over ALL experts (fp32, expf); the choice is made on score + correction (a bias
+// that steers the load and never reaches the weights; ties go to the lower index); the weights are the chosen experts'
+// scores over their sum.  One wave per token; lane l looks at experts l, l + 64, ...
+__global__ __launch_bounds__(256) void moe_route_softmax_kernel(int* __restrict__ sel, float* __restrict__ wt,
+                                                                const float* __restrict__ logits,
+                                                                const float* __restrict__ correction, int T, int E, int top) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  const float* z = logits + (long)t * E;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
+  float den = 0.f;
+  for (int e = lane; e < E; e += 64) den += expf(z[e] - mx);
+  den = wave_sum(den);
+  int prev_i = -1;
+  float prev_c = INFINITY, tot = 0.f;
+  for (int k = 0; k < top; ++k) {
+    // candidates come after (prev_c, prev_i) in the order "choice score descending, index ascending"
+    float best = -INFINITY, best_s = 0.f;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float s = expf(z[e] - mx) / den;
+      const float c = s + (correction ? correction[e] : 0.f);
+      const bool after = c < prev_c || (c == prev_c && e > prev_i);
+      if (after && (c > best || (c == best && e < bi))) { best = c; bi = e; best_s = s; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64), os = __shfl_xor(best_s, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; best_s = os; }
+    }
+    if (bi >= E) { bi = 0; best = -INFINITY; best_s = 0.f; }      // no candidate left (scores that are not numbers)
+    if (lane == 0) { sel[(long)t * top + k] = bi; wt[(long)t * top + k] = best_s; }
+    tot += best_s;
+    prev_c = best; prev_i = bi;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) wt[(long)t * top + k] = wt[(long)t * top + k] / (tot + 1e-20f);
+}
+
 // single workgroup: counts per expert (LDS atomics), row offsets, tile list, then every pair's row
 __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ pos_of, int* __restrict__ tiles,
                                                         const int* __restrict__ sel, int pairs, int E, int max_tiles, int TR) {
@@ -120,7 +165,7 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(typename El<P>::type* 
                                                           const typename El<P>::type* __restrict__ h, const float* __restrict__ wt,
                                                           const int* __restrict__ pos_of, int W, int top) {
   const int pr = blockIdx.x, t = pr / top;
-  const float wv = wt[pr];
+  const float wv = wt ? wt[pr] : 1.f;
   const long dst = (long)pos_of[pr] * W;
   for (int c = threadIdx.x; c < W; c += 256) stf<P>(xs + dst + c, wv * ldf<P>(h + (long)t * W + c));
 }
@@ -131,6 +176,17 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ y,
   for (int c = threadIdx.x; c < W; c += 256) {
     float a = add ? y[(long)t * W + c] : 0.f;
     for (int k = 0; k < top; ++k) a += ye[(long)pos_of[(long)t * top + k] * W + c];
+    y[(long)t * W + c] = a;
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_weighted_kernel(float* __restrict__ y, const float* __restrict__ ye,
+                                                                   const float* __restrict__ wt, const int* __restrict__ pos_of,
+                                                                   int W, int top, int add) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float a = add ? y[(long)t * W + c] : 0.f;
+    for (int k = 0; k < top; ++k) a += wt[(long)t * top + k] * ye[(long)pos_of[(long)t * top + k] * W + c];
     y[(long)t * W + c] = a;
   }
 }
@@ -166,7 +222,7 @@ extern "C" int umb_moe_plan(int* pos_of, int* tiles, const int* sel, int T, int 
 
 extern "C" int umb_moe_scatter(void* xs, const void* h, const float* wt, const int* pos_of, int T, int W, int top, int dtype,
                                hipStream_t st) {
-  if (T < 1 || W < 1 || top < 1 || !xs || !h || !wt || !pos_of) return UMB_EINVAL;
+  if (T < 1 || W < 1 || top < 1 || !xs || !h || !pos_of) return UMB_EINVAL;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
     hipLaunchKernelGGL(moe_scatter_kernel<P>, dim3(T * top), dim3(256), 0, st, (E*)xs, (const E*)h, wt, pos_of, W, top);
@@ -178,6 +234,22 @@ extern "C" int umb_moe_scatter(void* xs, const void* h, const float* wt, const i
 extern "C" int umb_moe_combine(float* y, const float* ye, const int* pos_of, int T, int W, int top, int add, hipStream_t st) {
   if (T < 1 || W < 1 || top < 1 || !y || !ye || !pos_of) return UMB_EINVAL;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, ye, pos_of, W, top, add);
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_moe_route_softmax(int* sel, float* wt, const float* logits, const float* correction, int T, int E, int top,
+                                     hipStream_t st) {
+  if (T < 1 || E < 1 || top < 1 || top > E || !sel || !wt || !logits) return UMB_EINVAL;
+  hipLaunchKernelGGL(moe_route_softmax_kernel, dim3((T + 3) / 4), dim3(256), 0, st, sel, wt, logits, correction, T, E, top);
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_moe_combine_weighted(float* y, const float* ye, const float* wt, const int* pos_of, int T, int W, int top,
+                                        int add, hipStream_t st) {
+  if (T < 1 || W < 1 || top < 1 || !y || !ye || !wt || !pos_of) return UMB_EINVAL;
+  hipLaunchKernelGGL(moe_combine_weighted_kernel, dim3(T), dim3(256), 0, st, y, ye, wt, pos_of, W, top, add);
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }

@@ -40,9 +40,14 @@ constexpr int GLA_COLS = 16;     // value columns per workgroup (4 per wave)
 // through a double-buffered LDS tile -- the global loads of chunk c + 1 are in flight while chunk c is consumed from LDS.
 // V4: D, Dv and the row stride of proj are multiples of 4 -> the staging moves 16-byte pieces (a quarter of the address
 // arithmetic, which is what this issue-bound kernel spends its time on).
+// Operand placement is general: q and k rows hold groups of D shared by `hpg` consecutive heads each (1: a group per head),
+// and the decay is per key channel (alpha [T][H D]) or, with aph, one number per head (alpha [T][H]) that fills the staged
+// row -- the state-space layers with a scalar decay per head run on the same kernel.
 template <int NR, bool V4>
 __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, float* __restrict__ state,
-                                                       const float* __restrict__ proj, int ld, const float* __restrict__ alpha,
+                                                       const float* __restrict__ qp, int ldq, const float* __restrict__ kp,
+                                                       int ldk, const float* __restrict__ vp, int ldv,
+                                                       const float* __restrict__ alpha, int aph, int hpg,
                                                        const int* __restrict__ seq_slot, const int* __restrict__ seq_row0,
                                                        const int* __restrict__ seq_pos0, const int* __restrict__ seq_len, int H,
                                                        int D, int Dv, float qscale) {
@@ -51,7 +56,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, fl
   constexpr int STG = (3 * NR + 1 + VW - 1) / VW;       // staged pieces per thread: TC (3 D + 16) / 256 <= 3 NR + 1 floats
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15;
   const int cbase = blockIdx.x * GLA_COLS, cl = wave * 4 + (lane >> 4), c = cbase + cl;
-  const int h = blockIdx.y, b = blockIdx.z;
+  const int h = blockIdx.y, b = blockIdx.z, hq = h / hpg;
   const int n = seq_len[b];
   if (n <= 0) return;
   const bool c_ok = c < Dv;
@@ -87,11 +92,19 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, fl
       const long row = row0 + t;
       int vc = cbase + ci - 3 * D;
       vc = vc + VW <= Dv ? vc : Dv - VW;
-      const float* src = ci < D ? alpha + row * HD + (long)h * D + ci
-                       : ci < 2 * D ? proj + row * ld + HD + (long)h * D + (ci - D)
-                       : ci < 3 * D ? proj + row * ld + (long)h * D + (ci - 2 * D)
-                                    : proj + row * ld + 2L * HD + (long)h * Dv + vc;
+      const bool is_a = ci < D;
+      const float* src = (is_a && !aph) ? alpha + row * HD + (long)h * D + ci
+                       : ci < 2 * D ? kp + row * ldk + (long)hq * D + (is_a ? ci : ci - D)
+                       : ci < 3 * D ? qp + row * ldq + (long)hq * D + (ci - 2 * D)
+                                    : vp + row * ldv + (long)h * Dv + vc;
       stage[e] = *reinterpret_cast<const piece*>(src);
+      if (aph) {                                        // uniform: one decay per head fills the alpha part of the row
+        const float a = alpha[row * H + h];
+        if (is_a) {
+          if constexpr (V4) stage[e] = piece{a, a, a, a};
+          else stage[e] = a;
+        }
+      }
     }
   };
   auto stash = [&](float* buf) {
@@ -212,19 +225,22 @@ extern "C" int umb_gla_decay(float* alpha, const float* proj, int ld, int a_col,
   return UMB_OK;
 }
 
-extern "C" int umb_gla_scan(float* o, float* state, const float* proj, int ld, const float* alpha, const int* seq_slot,
-                            const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int H, int D, int Dv,
-                            float qscale, hipStream_t st) {
-  if (B < 1 || H < 1 || D < 1 || D > 16 * GLA_MAXR || Dv < 1 || !o || !state || !proj || !alpha) return UMB_EINVAL;
+extern "C" int umb_lin_scan(float* o, float* state, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                            const float* alpha, int alpha_per_head, int qk_heads, const int* seq_slot, const int* seq_row0,
+                            const int* seq_pos0, const int* seq_len, int B, int H, int D, int Dv, float qscale, hipStream_t st) {
+  if (B < 1 || H < 1 || D < 1 || D > 16 * GLA_MAXR || Dv < 1 || qk_heads < 1 || H % qk_heads || !o || !state || !q || !k || !v ||
+      !alpha || ldq < qk_heads * D || ldk < qk_heads * D || ldv < H * Dv)
+    return UMB_EINVAL;
   const dim3 grid((Dv + GLA_COLS - 1) / GLA_COLS, H, B);
-  const int nr = (D + 15) / 16;
+  const int nr = (D + 15) / 16, aph = alpha_per_head ? 1 : 0, hpg = H / qk_heads;
   const size_t lds = 2 * (size_t)GLA_TC * (3 * D + GLA_COLS) * sizeof(float);
-  const bool v4 = D % 4 == 0 && Dv % 4 == 0 && ld % 4 == 0;
+  const bool v4 = D % 4 == 0 && Dv % 4 == 0 && ldq % 4 == 0 && ldk % 4 == 0 && ldv % 4 == 0 &&
+                  ((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (aph ? 0 : (uintptr_t)alpha)) % 16 == 0;
 #define GLA_SCAN_LAUNCH(NR, V4)                                                                                           \
   do {                                                                                                                    \
     if (ensure_dynamic_lds<gla_scan_kernel<NR, V4>>(lds) != UMB_OK) return UMB_EHIP;                                      \
-    hipLaunchKernelGGL((gla_scan_kernel<NR, V4>), grid, dim3(256), lds, st, o, state, proj, ld, alpha, seq_slot, seq_row0, \
-                       seq_pos0, seq_len, H, D, Dv, qscale);                                                              \
+    hipLaunchKernelGGL((gla_scan_kernel<NR, V4>), grid, dim3(256), lds, st, o, state, q, ldq, k, ldk, v, ldv, alpha, aph, \
+                       hpg, seq_slot, seq_row0, seq_pos0, seq_len, H, D, Dv, qscale);                                      \
   } while (0)
 #define GLA_SCAN_CASE(NR)                                                                                                 \
   case NR:                                                                                                                \
@@ -240,6 +256,14 @@ extern "C" int umb_gla_scan(float* o, float* state, const float* proj, int ld, c
 #undef GLA_SCAN_LAUNCH
   UMB_LAUNCH_CHECK();
   return UMB_OK;
+}
+
+extern "C" int umb_gla_scan(float* o, float* state, const float* proj, int ld, const float* alpha, const int* seq_slot,
+                            const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int H, int D, int Dv,
+                            float qscale, hipStream_t st) {
+  if (!proj || H < 1 || D < 1 || Dv < 1 || ld < 2 * H * D + H * Dv) return UMB_EINVAL;
+  return umb_lin_scan(o, state, proj, ld, proj + (long)H * D, ld, proj + 2L * H * D, ld, alpha, 0, H, seq_slot, seq_row0, seq_pos0,
+                      seq_len, B, H, D, Dv, qscale, st);
 }
 
 extern "C" int umb_gla_gate(void* out, const float* o, const float* proj, int ld, int g_col, const void* w, int T, int H, int Dv,

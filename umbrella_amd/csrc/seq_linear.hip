@@ -56,7 +56,7 @@ template <> __device__ __forceinline__ f32x4 mma8<F32>(const Frag8<F32>& a, cons
   return c;
 }
 
-enum { EPI_F32 = 0, EPI_DT = 1, EPI_SILU_MUL = 2, EPI_GATE = 3 };
+enum { EPI_F32 = 0, EPI_DT = 1, EPI_SILU_MUL = 2, EPI_GATE = 3, EPI_RELU2 = 4 };
 
 // Where a launch departs from the dense [T][K] x [N][K] problem: row strides of x and out, a batch of independent problems
 // along blockIdx.z (element strides sx / sw / so), or token tiles read from device memory (grouped: tile blockIdx.y is
@@ -184,6 +184,9 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
         stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, siluf_(s) * u);
       } else if (epi == EPI_DT) {
         stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, s);
+      } else if (epi == EPI_RELU2) {
+        const float rl = fmaxf(s, 0.f);
+        stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, rl * rl);
       } else if (epi == EPI_GATE) {
         stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, s / (1.f + expf(-gate[(long)t * ext.ldg + n])));
       } else {
@@ -301,6 +304,9 @@ __global__ __launch_bounds__(256) void seq_linear_wide_kernel(void* __restrict__
           reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(siluf_(sv) * uv);
         } else if (epi == EPI_DT) {
           reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(sv);
+        } else if (epi == EPI_RELU2) {
+          const float rl = fmaxf(sv, 0.f);
+          reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(rl * rl);
         } else {
           reinterpret_cast<float*>(out_)[obase + (long)t * N + n] = sv;
         }
@@ -361,7 +367,7 @@ static int launch_vec(void* out, const void* x, const void* w, const void* bias,
 
 extern "C" int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, int dtype,
                               hipStream_t st) {
-  if (T < 1 || N < 1 || K < 1 || epi < 0 || epi > 2 || !out || !x || !w) return UMB_EINVAL;
+  if (T < 1 || N < 1 || K < 1 || epi < 0 || (epi > 2 && epi != EPI_RELU2) || !out || !x || !w) return UMB_EINVAL;
   if (epi == EPI_SILU_MUL) {
     if (N & 1) return UMB_EINVAL;
     N >>= 1;                                   // rows of each half
@@ -390,7 +396,7 @@ extern "C" int umb_seq_linear_batched(void* out, const void* x, const void* w, i
 
 extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows,
                                       long gs, int N, int K, int epi, int dtype, hipStream_t st) {
-  if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || epi > 2 || !out || !x || !w || !tiles ||
+  if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || (epi > 2 && epi != EPI_RELU2) || !out || !x || !w || !tiles ||
       (tile_rows != 16 && tile_rows != 64 && tile_rows != 128))
     return UMB_EINVAL;
   if (epi == EPI_SILU_MUL) {

@@ -6,6 +6,11 @@
 //     attention: proj GEMM | rope + unit-norm + append | pool | attend (matrix pipe for prompts) | out GEMM | seam | gate-up GEMM (SiLU*up epilogue) |
 //                down GEMM | seam
 //     GLA:       proj GEMM | decay | scan | head norm * SiLU gate | out GEMM | seam (| feed-forward as above)
+//     minGRU:    proj GEMM ([z | x | g], biases in the GEMM) | scan with the output gate | out GEMM | seam
+//     attention beside a state-space layer (both read the same input, one fused proj GEMM, one out GEMM over [a | b]):
+//                norms + temperature + append | attend  ||  convolution + dt + decay | state ring | scan | gate + norm
+// Models with several residual streams (UmbSeqModel.streams >= 1) use the stream seam instead: write of the sublayer behind
+// it and read (combination + norm) of the one ahead in one launch.
 // Nothing here depends on the host between launches: a step can be captured into a hipGraph.
 #include "seq_common.h"
 
@@ -52,8 +57,10 @@ static int seam(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s,
 // feed-forward of ws->h into ws->y (fp32)
 static int feed_forward(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSeqWork* ws, const UmbSeqStep* s, hipStream_t st) {
   const int T = s->T, W = m->W, dt = m->dtype;
+  // the activation lives in the first product's epilogue: silu(gate) * up over stacked [gate; up], or relu(up)^2
+  const int epi = ly.act_kind == UMB_ACT_RELU2 ? 4 : 2, stack = ly.act_kind == UMB_ACT_RELU2 ? 1 : 2;
   if (ly.ff_kind == UMB_FF_GATED) {
-    SEQ_TRY(lin(ly.gu, ws->act, ws->h, T, 2, dt, st));
+    SEQ_TRY(lin(ly.gu, ws->act, ws->h, T, epi, dt, st));
     return lin(ly.down, ws->y, ws->act, T, 0, dt, st);
   }
   if (ly.ff_kind == UMB_FF_POLYNORM) {
@@ -74,18 +81,63 @@ static int feed_forward(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
     const int max_tiles = (int)((pairs + tr - 1) / tr) + E;
     if (max_tiles > ws->moe_max_tiles) return UMB_EINVAL;
     if (ly.s_gu.w) {                                                           // the shared expert sees every token
-      SEQ_TRY(lin(ly.s_gu, ws->act, ws->h, T, 2, dt, st));
+      SEQ_TRY(lin(ly.s_gu, ws->act, ws->h, T, epi, dt, st));
       SEQ_TRY(lin(ly.s_down, ws->y, ws->act, T, 0, dt, st));
     }
     SEQ_TRY(lin(ly.router, ws->proj, ws->h, T, 0, dt, st));
-    SEQ_TRY(umb_moe_route(ws->moe_sel, ws->moe_wt, ws->proj, T, E, top, st));
+    // sigmoid routing weighs the expert's input, softmax routing its output
+    const bool w_out = ly.route_kind == UMB_ROUTE_SOFTMAX_OUT;
+    if (w_out) SEQ_TRY(umb_moe_route_softmax(ws->moe_sel, ws->moe_wt, ws->proj, ly.correction, T, E, top, st));
+    else SEQ_TRY(umb_moe_route(ws->moe_sel, ws->moe_wt, ws->proj, T, E, top, st));
     SEQ_TRY(umb_moe_plan(ws->moe_pos, ws->moe_tiles, ws->moe_sel, T, E, top, max_tiles, tr, st));
-    SEQ_TRY(umb_moe_scatter(ws->moe_xs, ws->h, ws->moe_wt, ws->moe_pos, T, W, top, dt, st));
-    SEQ_TRY(umb_seq_linear_grouped(ws->moe_act, ws->moe_xs, ly.e_gu, ws->moe_tiles, max_tiles, tr, 2L * F * W, 2 * F, W, 2, dt, st));
+    SEQ_TRY(umb_moe_scatter(ws->moe_xs, ws->h, w_out ? nullptr : ws->moe_wt, ws->moe_pos, T, W, top, dt, st));
+    SEQ_TRY(umb_seq_linear_grouped(ws->moe_act, ws->moe_xs, ly.e_gu, ws->moe_tiles, max_tiles, tr, (long)stack * F * W, stack * F, W,
+                                   epi, dt, st));
     SEQ_TRY(umb_seq_linear_grouped(ws->moe_y, ws->moe_act, ly.e_down, ws->moe_tiles, max_tiles, tr, (long)W * F, W, F, 0, dt, st));
+    if (w_out) return umb_moe_combine_weighted(ws->y, ws->moe_y, ws->moe_wt, ws->moe_pos, T, W, top, ly.s_gu.w ? 1 : 0, st);
     return umb_moe_combine(ws->y, ws->moe_y, ws->moe_pos, T, W, top, ly.s_gu.w ? 1 : 0, st);
   }
   return UMB_EINVAL;
+}
+
+// minGRU: proj = [z | x | g] with the biases of z and x added by the product; the scan applies the output gate
+static int mix_mingru(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSeqWork* ws, const UmbSeqStep* s, hipStream_t st) {
+  const int Wm = ly.dim;
+  if (ly.proj.N != 3 * Wm || !ly.state || ly.out.K != Wm) return UMB_EINVAL;
+  return umb_mingru_scan(ws->mix, ly.state, ws->proj, 3 * Wm, 0, Wm, 2 * Wm, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B,
+                         Wm, m->dtype, st);
+}
+
+// softmax attention with a distance bias beside a state-space layer; both read the projection of the same input and write
+// their halves of the row that the one output projection reads: [scale_a * attention | scale_b * state space]
+static int mix_attn_ssd(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSeqWork* ws, const UmbSeqStep* s, hipStream_t st) {
+  const int T = s->T, dt = m->dtype, ld = ly.proj.N;
+  const int H = ly.heads, G = ly.kv_heads, D = ly.dim, E = ly.vdim;
+  const int sH = ly.s_heads, sDv = ly.s_vdim, N = ly.s_state, sG = ly.s_groups;
+  if (H < 1 || G < 1 || sH < 1 || sG < 1) return UMB_EINVAL;
+  const int gate_col = H * D + G * D + G * E, col0 = gate_col + H;
+  const int inner = sH * sDv, C = inner + 2 * sG * N, lds = C + inner, ldo = H * E + inner;
+  if (ld != col0 + 2 * inner + 2 * sG * N + sH || ly.out.K != ldo || !ly.state) return UMB_EINVAL;
+  float* q = ws->aux;                                        // [T][H D] | [T][lds] | [T][sH]
+  float* sx = q + (size_t)T * H * D;
+  float* alpha = sx + (size_t)T * lds;
+  SEQ_TRY(umb_bsa_prep(q, &ly.kv, ws->proj, ld, ly.q_norm, ly.k_norm, s->pos, s->slot, T, H, G, D, E, ly.temp_coef, ly.temp_every,
+                       m->eps, dt, st));
+  if (s->max_len >= 16 && umb_bsa_attend_tiled_ok(H, G, D, E, dt))
+    SEQ_TRY(umb_bsa_attend_tiled(ws->mix, ldo, q, &ly.kv, ws->proj, ld, gate_col, ly.dist_bias, ly.n_dist, s->seq_slot, s->seq_row0,
+                                 s->seq_pos0, s->seq_len, s->B, s->max_len, H, G, D, E, ly.window, ly.scale, ly.mix_scale_a, dt, st));
+  else
+    SEQ_TRY(umb_bsa_attend(ws->mix, ldo, q, &ly.kv, ws->proj, ld, gate_col, ly.dist_bias, ly.n_dist, s->pos, s->slot, T, H, G, D, E,
+                           ly.window, ly.scale, ly.mix_scale_a, dt, st));
+  SEQ_TRY(umb_ssd_prep(sx, lds, alpha, ws->proj, ld, col0, ly.s_conv, ly.s_conv_b, ly.s_conv_state, ly.s_dt_bias, ly.s_a_log, s->pos,
+                       s->slot, T, sH, sDv, sG, N, ly.s_taps, dt, st));
+  SEQ_TRY(umb_ssd_conv_update(ly.s_conv_state, ws->proj, ld, col0 + inner, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B,
+                              C, ly.s_taps, st));
+  SEQ_TRY(umb_lin_scan(ws->o, ly.state, sx + inner + sG * N, lds, sx + inner, lds, sx, lds, alpha, 1, sG, s->seq_slot, s->seq_row0,
+                       s->seq_pos0, s->seq_len, s->B, sH, N, sDv, 1.f, st));
+  void* right = static_cast<char*>(ws->mix) + (size_t)H * E * seq_elem_bytes(dt);
+  return umb_ssd_gate(right, ldo, ws->o, sx, lds, C, ws->proj, ld, col0, ly.s_d, ly.s_norm, T, sH, sDv, ly.s_norm_groups, m->eps,
+                      ly.mix_scale_b, dt, st);
 }
 
 extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s, hipStream_t st) {
@@ -93,7 +145,13 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
     return UMB_EINVAL;
   const int T = s->T, W = m->W, dt = m->dtype, groups = m->groups;
   const float eps = m->eps;
-  if (m->layers[0].norm1)
+  const bool hyper = m->streams >= 1;          // several residual streams: norms in front only, stream seams
+  const int S = m->streams;
+  if (hyper) {
+    if (!m->layers[0].norm1) return UMB_EINVAL;
+    SEQ_TRY(umb_hc_embed(ws->x, ws->h, m->embed, s->tokens, m->embed_scale, m->layers[0].hc1_in, m->layers[0].norm1,
+                         m->norm_offset, T, W, m->V, S, eps, dt, st));
+  } else if (m->layers[0].norm1)
     SEQ_TRY(umb_seq_embed_norm(ws->x, ws->h, m->embed, s->tokens, m->layers[0].norm1, T, W, m->V, groups, eps, dt, st));
   else
     SEQ_TRY(umb_seq_embed(ws->x, m->embed, s->tokens, m->embed_scale, T, W, m->V, dt, st));
@@ -102,7 +160,7 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
     const UmbSeqLayer& ly = m->layers[l];
     const UmbSeqLayer* nl = l + 1 < m->L ? &m->layers[l + 1] : nullptr;
     const int ld = ly.proj.N;
-    SEQ_TRY(sublayer_input(m, ws, s, ly.norm1, ly.canon1, ly.canon_state1, h_ready, st));
+    if (!hyper) SEQ_TRY(sublayer_input(m, ws, s, ly.norm1, ly.canon1, ly.canon_state1, h_ready, st));
     SEQ_TRY(lin(ly.proj, ws->proj, ws->h, T, 0, dt, st));
     if (ly.kind == UMB_MIX_POOLED_WINDOW) {
       const int H = ly.heads, G = ly.kv_heads, D = ly.dim;
@@ -143,10 +201,29 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
         SEQ_TRY(umb_lat_attend(ws->act, ws->aux, &ly.kv, ly.sink, s->pos, s->slot, T, H, Rc, R, ly.window, ly.scale, dt, st));
       SEQ_TRY(umb_seq_linear_batched(ws->mix, ws->act, ly.uv, T, Dv, Rc, H * Rc, H * Dv, H, Rc, (long)Dv * Rc, Dv, 3,
                                      ws->proj + Rq + Dk, ld, Dv, dt, st));
+    } else if (ly.kind == UMB_MIX_MINGRU) {
+      SEQ_TRY(mix_mingru(m, ly, ws, s, st));
+    } else if (ly.kind == UMB_MIX_ATTN_SSD) {
+      SEQ_TRY(mix_attn_ssd(m, ly, ws, s, st));
     } else {
       return UMB_EINVAL;
     }
     SEQ_TRY(lin(ly.out, ws->y, ws->mix, T, 0, dt, st));
+    if (hyper) {
+      // write of this sublayer and read of the next one (the feed-forward, the next layer's mixer, or nothing) in one launch
+      const float* in2 = ly.has_mlp ? ly.hc2_in : (nl ? nl->hc1_in : nullptr);
+      const void* w2 = ly.has_mlp ? ly.norm2 : (nl ? nl->norm1 : nullptr);
+      if ((ly.has_mlp || nl) && !w2) return UMB_EINVAL;
+      SEQ_TRY(umb_hc_seam(ws->x, ws->h, ws->y, ly.hc1_mix, ly.hc1_out, m->resid_mult, in2, w2, m->norm_offset, T, W, S, eps, dt, st));
+      if (ly.has_mlp) {
+        SEQ_TRY(feed_forward(m, ly, ws, s, st));
+        if (nl && !nl->norm1) return UMB_EINVAL;
+        SEQ_TRY(umb_hc_seam(ws->x, ws->h, ws->y, ly.hc2_mix, ly.hc2_out, m->resid_mult, nl ? nl->hc1_in : nullptr,
+                            nl ? nl->norm1 : nullptr, m->norm_offset, T, W, S, eps, dt, st));
+      }
+      if (s->trace) SEQ_TRY(umb_hc_read(s->trace + (long)l * T * W, nullptr, ws->x, nullptr, nullptr, nullptr, 0.f, T, W, S, eps, dt, st));
+      continue;
+    }
     const void* next = ly.has_mlp ? ly.norm2 : first_norm_of(m, l + 1);
     SEQ_TRY(seam(m, ws, s, ly.norm1b, next, ly.has_mlp ? ly.canon2 : (nl ? nl->canon1 : nullptr),
                  ly.has_mlp ? ly.canon_state2 : (nl ? nl->canon_state1 : nullptr), &h_ready, st));
@@ -162,8 +239,11 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
     }
   }
   if (s->R > 0) {
-    // final norm of the wanted rows only, then the head
-    SEQ_TRY(umb_seq_group_norm(nullptr, ws->h, ws->x, s->logit_rows, m->final_norm, s->R, W, groups, eps, dt, st));
+    // final norm of the wanted rows only (of the sum of the streams, where there are several), then the head
+    if (hyper)
+      SEQ_TRY(umb_hc_read(nullptr, ws->h, ws->x, s->logit_rows, nullptr, m->final_norm, m->norm_offset, s->R, W, S, eps, dt, st));
+    else
+      SEQ_TRY(umb_seq_group_norm(nullptr, ws->h, ws->x, s->logit_rows, m->final_norm, s->R, W, groups, eps, dt, st));
     SEQ_TRY(lin(m->head, ws->logits, ws->h, s->R, 0, dt, st));
   }
   return UMB_OK;

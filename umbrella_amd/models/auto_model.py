@@ -15,12 +15,13 @@ from .config import KNOWN, read_architecture
 from .fidizen import Fidizen
 from .gitopel import Gitopel
 from .llama import Llama
+from .tomopel import Tomopel
 
 
 class AutoModelLM:
     # a local directory is resolved by the architecture its config.json names; directories that name none of these are
     # Hugging Face Llama / Qwen2 / Mistral checkpoints
-    _ARCHITECTURE_MAPPING = {"Gitopel": Gitopel, "Fidizen": Fidizen}
+    _ARCHITECTURE_MAPPING = {"Gitopel": Gitopel, "Fidizen": Fidizen, "Tomopel": Tomopel}
     _MODEL_MAPPING = {name: Llama for name in KNOWN}
     _OFFLOAD_MODEL_MAPPING = dict(_MODEL_MAPPING)
     _CUDAGRAPH_MODEL_MAPPING = dict(_MODEL_MAPPING)

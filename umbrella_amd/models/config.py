@@ -242,8 +242,51 @@ class LatentAttnCfg:
 
 
 @dataclass
+class MinGRUCfg:
+    """Minimal gated recurrence over ``dim`` channels, element by element: the gates read only the current token; one fp32
+    state per channel; a SiLU output gate.  (``heads`` / ``vdim`` describe the state to the cache manager.)"""
+    dim: int
+    heads: int = 1
+    vdim: int = 1
+    kind: str = "mingru"
+
+
+@dataclass
+class AttnSSDCfg:
+    """Two mixers side by side that read the same input and share one output projection over ``[a_scale * attention |
+    b_scale * state space]``.
+
+    Attention: causal softmax (``window`` 0: every earlier position), grouped query heads, unit-RMS q / k with a weight
+    shared by the heads, weightless unit-RMS values, a query temperature ``1 + temp_coef ln(floor((p + 1) / temp_every) + 1)``,
+    a learned bias per (distance bucket, head) -- ``bias_rows`` buckets: exact below half of them, logarithmic up to
+    ``bias_far`` -- and one sigmoid output gate per head.
+    State space: ``s_heads`` heads of ``s_vdim`` with an ``[s_state, s_vdim]`` fp32 state each, one decay per head, B / C
+    shared by ``s_groups`` groups of heads, a causal convolution of ``s_taps`` taps in front, a gated RMS norm in
+    ``s_norm_groups`` parts behind."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int
+    bias_rows: int
+    bias_far: float
+    temp_coef: float
+    temp_every: int
+    a_scale: float
+    s_heads: int
+    s_vdim: int
+    s_state: int
+    s_groups: int
+    s_norm_groups: int
+    s_taps: int
+    b_scale: float
+    kind: str = "attention_ssd"
+
+
+@dataclass
 class SeqLayerCfg:
-    mixer: object                    # PooledWindowAttnCfg | GLACfg | LatentAttnCfg
+    mixer: object                    # PooledWindowAttnCfg | GLACfg | LatentAttnCfg | MinGRUCfg | AttnSSDCfg
     ff: int = 0                      # width of the dense feed-forward; 0 = the layer has none (or has experts)
     ff_kind: str = "gated"           # "gated": W_down (silu(W_gate h) * W_up h); "polynorm": W_down polynorm(W_up h); "moe"
     experts: int = 0                 # "moe": routed experts, how many each token uses, their width, the shared expert's
@@ -251,6 +294,9 @@ class SeqLayerCfg:
     expert_ff: int = 0
     shared_ff: int = 0               # 0: no shared expert
     weights_of: int | None = None    # the layer uses that layer's tensors (with a cache and state of its own)
+    act: str = "silu_gated"          # "silu_gated": silu(W_gate h) * W_up h; "relu2": relu(W_up h)^2 (no gate) -- dense, experts, shared
+    route: str = "sigmoid_in"        # "sigmoid_in": sigmoid scores weigh the expert's input; "softmax_out": softmax scores,
+                                     # chosen with a correction added, renormalised over the chosen, weigh its output
 
     @property
     def has_ff(self) -> bool:
@@ -270,6 +316,10 @@ class SeqMixCfg:
     embed_scale: float = 1.0         # the embedding row is multiplied by it
     pre_norm: bool = True            # False: sublayers read the residual stream itself, only their output is normed
     canon_taps: int = 0              # > 0: every sublayer reads h + causal_conv(h) over this many positions (pre_norm False)
+    streams: int = 0                 # >= 1: that many residual streams with read / write / mix weights per sublayer (norms
+                                     # in front of the sublayers only); 0: one stream with the seams above
+    resid_mult: float = 1.0          # a sublayer's output is multiplied by it before it joins the residual (streams >= 1)
+    norm_offset: float = 0.0         # norm weights are stored around it: the factor is offset + w (streams >= 1)
 
     @property
     def num_hidden_layers(self):

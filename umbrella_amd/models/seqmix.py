@@ -1,9 +1,11 @@
 """Runtime of the sequence-mixer model family on the HIP path (libumbrella_seq.so, include/umbrella_seq.h).
 
-A model is a LIST of layers, each a token mixer -- windowed attention with pooled blocks, gated linear attention, or latent
-attention -- plus an optional feed-forward (gated SiLU, PolyNorm, or routed experts with a shared one).  A sublayer reads either
-a grouped RMS norm of the residual stream or the stream itself through a short causal convolution; its output is normed before
-it is added back.  A layer may use another layer's tensors with a cache and state of its own.  The list, every size and every
+A model is a LIST of layers, each a token mixer -- windowed attention with pooled blocks, gated linear attention, latent
+attention, a minimal gated recurrence, or softmax attention beside a state-space layer -- plus an optional feed-forward (gated
+SiLU, PolyNorm, or routed experts with a shared one).  A sublayer reads either a grouped RMS norm of the residual stream or the
+stream itself through a short causal convolution; its output is normed before it is added back; or (``streams >= 1``) the
+residual is several streams that every sublayer reads as one combination and writes back to all.  A layer may use another
+layer's tensors with a cache and state of its own.  The list, every size and every
 constant come from a ``SeqMixCfg`` (models/config.py); a design contributes a subclass that names its checkpoint tensors
 (models/gitopel.py, models/fidizen.py).
 
@@ -27,8 +29,10 @@ from ..attn.cache import PagedSeqCache
 from .base import LLMBase
 from .config import SeqMixCfg
 
-KIND_CODE = {"attention": 0, "gla": 1, "latent_attention": 2}
+KIND_CODE = {"attention": 0, "gla": 1, "latent_attention": 2, "mingru": 3, "attention_ssd": 4}
 FF_CODE = {"gated": 0, "polynorm": 1, "moe": 2}
+ACT_CODE = {"silu_gated": 0, "relu2": 1}
+ROUTE_CODE = {"sigmoid_in": 0, "softmax_out": 1}
 
 
 def _linear(w, b=None) -> UmbSeqLinear:
@@ -75,6 +79,7 @@ class SeqMixLM(LLMBase):
         dev, dt = self.device, self.dtype
         if self._state is not None:
             sd = self._state
+            self._names = set(sd.keys())
             return lambda name: sd[name].to(device=dev, dtype=dt if sd[name].is_floating_point() else None).contiguous()
         from safetensors import safe_open
         files = [os.path.join(self.model_name, f) for f in sorted(os.listdir(self.model_name)) if f.endswith(".safetensors")]
@@ -83,12 +88,17 @@ class SeqMixLM(LLMBase):
             with safe_open(f, "pt") as h:
                 for k in h.keys():
                     index[k] = f
+        self._names = set(index.keys())
 
         def get(name):
             with safe_open(index[name], "pt") as h:
                 t = h.get_tensor(name)
             return t.to(device=dev, dtype=dt if t.is_floating_point() else None).contiguous()
         return get
+
+    def has_tensor(self, name: str) -> bool:
+        """whether the checkpoint holds a tensor of that name (valid while ``alloc`` reads the weights)"""
+        return name in self._names
 
     def alloc(self, **kwargs):
         c, dev, dt = self.config, self.device, self.dtype
@@ -97,7 +107,7 @@ class SeqMixLM(LLMBase):
         self._top = self.top_tensors(get)
         assert tuple(self._top["embed"].shape) == (c.vocab_size, c.width), tuple(self._top["embed"].shape)
         L = len(c.layers)
-        self._tensors, kv_layers, state_layers, latent_layers, n_conv = [], [], [], [], 0
+        self._tensors, kv_layers, state_layers, latent_layers, n_conv, mixer_convs = [], [], [], [], 0, []
         for i, ly in enumerate(c.layers):
             if ly.weights_of is not None:
                 # the tensors of another layer (which must own its tensors), a cache and state of this layer's own
@@ -118,10 +128,20 @@ class SeqMixLM(LLMBase):
             elif m.kind == "latent_attention":
                 t["cache_index"] = len(latent_layers)
                 latent_layers.append(m.kv_rank + m.rot_dim)
+            elif m.kind == "mingru":
+                t["cache_index"] = len(state_layers)
+                state_layers.append((1, 1, m.dim))
+            elif m.kind == "attention_ssd":
+                if m.heads % m.kv_heads or m.s_heads % m.s_groups or (m.s_heads * m.s_vdim) % m.s_norm_groups:
+                    raise ValueError("heads / kv_heads, state-space heads / groups and inner width / norm groups must divide")
+                t["cache_index"], t["state_index"], t["mconv_index"] = len(kv_layers), len(state_layers), len(mixer_convs)
+                kv_layers.append((m.kv_heads, m.dim, 0, m.vdim))
+                state_layers.append((m.s_heads, m.s_state, m.s_vdim))
+                mixer_convs.append((m.s_taps, m.s_heads * m.s_vdim + 2 * m.s_groups * m.s_state))
             else:
                 t["cache_index"] = len(state_layers)
                 state_layers.append((m.heads, m.dim, m.vdim))
-            if m.kind != "gla" and "rot_freq" not in t:
+            if m.kind in ("attention", "latent_attention") and "rot_freq" not in t:
                 i2 = torch.arange(m.rot_dims // 2, dtype=torch.float32)
                 t["rot_freq"] = (m.rot_base ** (-2 * i2 / m.rot_dims)).to(dev) if m.rot_dims else None     # fp32 frequencies
             if c.canon_taps > 0:
@@ -129,7 +149,8 @@ class SeqMixLM(LLMBase):
                 n_conv += 2 if ly.has_ff else 1
             self._tensors.append(t)
         self.kv_cache = PagedSeqCache(kv_layers, state_layers, self.max_tokens, self.batch_size, dev, dt, page=self.page_size,
-                                      latent_layers=latent_layers, conv_states=n_conv, conv_taps=c.canon_taps, width=c.width)
+                                      latent_layers=latent_layers, conv_states=n_conv, conv_taps=c.canon_taps, width=c.width,
+                                      mixer_convs=mixer_convs)
         self._layer_structs = (UmbSeqLayer * L)()
         for i, (ly, t) in enumerate(zip(c.layers, self._tensors)):
             s, m = self._layer_structs[i], ly.mixer
@@ -137,7 +158,12 @@ class SeqMixLM(LLMBase):
             s.ff_kind = FF_CODE[ly.ff_kind]
             s.proj, s.out = _linear(t["proj_w"], t.get("proj_b")), _linear(t["out_w"], t.get("out_b"))
             s.norm1 = t["norm1"].data_ptr() if t.get("norm1") is not None else None
-            s.norm1b = t["norm1b"].data_ptr()
+            s.norm1b = t["norm1b"].data_ptr() if t.get("norm1b") is not None else None
+            s.act_kind, s.route_kind = ACT_CODE[ly.act], ROUTE_CODE[ly.route]
+            for q in ("hc1", "hc2"):                              # read / write / mix weights of the residual streams (fp32)
+                for part in ("in", "out", "mix"):
+                    v = t.get(f"{q}_{part}")
+                    setattr(s, f"{q}_{part}", v.data_ptr() if v is not None else None)
             if c.canon_taps > 0:
                 s.canon1, s.canon_state1 = t["canon1"].data_ptr(), self.kv_cache.conv[t["conv_index"]].data_ptr()
             if m.kind == "attention":
@@ -153,18 +179,37 @@ class SeqMixLM(LLMBase):
                 s.dq_norm, s.dkv_norm = t["dq_norm"].data_ptr(), t["dkv_norm"].data_ptr()
                 s.sink = t["sink"].data_ptr() if t.get("sink") is not None else None
                 s.kv = self.kv_cache.latent_struct(t["cache_index"])
+            elif m.kind == "mingru":
+                s.state = self.kv_cache.state[t["cache_index"]].data_ptr()
+            elif m.kind == "attention_ssd":
+                s.kv_heads, s.scale, s.window = m.kv_heads, m.scale, (m.window if m.window > 0 else 2 ** 30)
+                s.q_norm = t["q_norm"].data_ptr() if t.get("q_norm") is not None else None
+                s.k_norm = t["k_norm"].data_ptr() if t.get("k_norm") is not None else None
+                if t.get("dist_bias") is not None:                 # fp32 [heads][n_dist], indexed by the clamped distance
+                    s.dist_bias, s.n_dist = t["dist_bias"].data_ptr(), t["dist_bias"].shape[1]
+                s.temp_coef, s.temp_every = float(m.temp_coef), int(m.temp_every)
+                s.mix_scale_a, s.mix_scale_b = float(m.a_scale), float(m.b_scale)
+                s.s_heads, s.s_vdim, s.s_state, s.s_groups = m.s_heads, m.s_vdim, m.s_state, m.s_groups
+                s.s_norm_groups, s.s_taps = m.s_norm_groups, m.s_taps
+                s.s_conv, s.s_norm = t["s_conv"].data_ptr(), t["s_norm"].data_ptr()
+                s.s_conv_b = t["s_conv_b"].data_ptr() if t.get("s_conv_b") is not None else None
+                s.s_dt_bias, s.s_a_log, s.s_d = t["s_dt_bias"].data_ptr(), t["s_a_log"].data_ptr(), t["s_d"].data_ptr()
+                s.s_conv_state = self.kv_cache.mixer_conv[t["mconv_index"]].data_ptr()
+                s.kv = self.kv_cache.struct(t["cache_index"])
+                s.state = self.kv_cache.state[t["state_index"]].data_ptr()
             else:
                 s.rank, s.tau, s.qscale = m.rank, m.tau, float(m.dim) ** -0.5
                 s.a2, s.head_norm = _linear(t["a2_w"], t["a2_b"]), t["head_norm"].data_ptr()
                 s.state = self.kv_cache.state[t["cache_index"]].data_ptr()
             if ly.has_ff:
                 s.norm2 = t["norm2"].data_ptr() if t.get("norm2") is not None else None
-                s.norm2b = t["norm2b"].data_ptr()
+                s.norm2b = t["norm2b"].data_ptr() if t.get("norm2b") is not None else None
                 if c.canon_taps > 0:
                     s.canon2, s.canon_state2 = t["canon2"].data_ptr(), self.kv_cache.conv[t["conv_index"] + 1].data_ptr()
                 if ly.ff_kind == "moe":
                     s.experts, s.top, s.expert_ff, s.shared_ff = ly.experts, ly.top, ly.expert_ff, ly.shared_ff
                     s.router, s.e_gu, s.e_down = _linear(t["router_w"]), t["e_gu"].data_ptr(), t["e_down"].data_ptr()
+                    s.correction = t["correction"].data_ptr() if t.get("correction") is not None else None
                     if ly.shared_ff:
                         s.s_gu, s.s_down = _linear(t["s_gu_w"]), _linear(t["s_down_w"])
                 else:
@@ -174,6 +219,7 @@ class SeqMixLM(LLMBase):
         mdl = self._m = UmbSeqModel()
         mdl.dtype, mdl.L, mdl.W, mdl.V, mdl.groups, mdl.eps = _lib.seq_dtype_code(dt), L, c.width, c.vocab_size, c.norm_groups, c.norm_eps
         mdl.embed_scale, mdl.canon_taps = float(c.embed_scale), int(c.canon_taps)
+        mdl.streams, mdl.resid_mult, mdl.norm_offset = int(c.streams), float(c.resid_mult), float(c.norm_offset)
         mdl.embed, mdl.final_norm, mdl.head = self._top["embed"].data_ptr(), self._top["final_norm"].data_ptr(), _linear(self._top["head"])
         mdl.layers = C.cast(self._layer_structs, C.POINTER(UmbSeqLayer))
         self.reserve(self.max_step_tokens or 256)
@@ -203,6 +249,12 @@ class SeqMixLM(LLMBase):
                 # aux: queries carried into the latent space
                 ask(act=max(m.q_rank, m.heads * m.kv_rank), o=m.heads * (m.dim + m.rot_dim), mix=m.heads * max(m.dim, m.vdim),
                     aux=m.heads * (m.kv_rank + m.rot_dim))
+            elif m.kind == "mingru":
+                ask(mix=m.dim)
+            elif m.kind == "attention_ssd":
+                # aux: queries | convolved [dt x | B | C | x] | decays; o: the scan's read-out; mix: [attention | state space]
+                inner = m.s_heads * m.s_vdim
+                ask(aux=m.heads * m.dim + 2 * inner + 2 * m.s_groups * m.s_state + m.s_heads, o=inner, mix=m.heads * m.vdim + inner)
             else:
                 ask(aux=m.heads * m.dim, o=m.heads * m.vdim, mix=m.heads * m.vdim)
             if ly.ff_kind == "moe":
@@ -212,7 +264,7 @@ class SeqMixLM(LLMBase):
                 ask(act=ly.ff, proj=ly.ff if ly.ff_kind == "polynorm" else 1)
         f32, i32 = torch.float32, torch.int32
         b = self._bufs = dict(
-            x=torch.zeros(T, c.width, dtype=f32, device=dev), h=torch.zeros(T, c.width, dtype=dt, device=dev),
+            x=torch.zeros(T, max(1, c.streams) * c.width, dtype=f32, device=dev), h=torch.zeros(T, c.width, dtype=dt, device=dev),
             proj=torch.zeros(T, need["proj"], dtype=f32, device=dev), aux=torch.zeros(T, need["aux"], dtype=f32, device=dev),
             o=torch.zeros(T, need["o"], dtype=f32, device=dev), mix=torch.zeros(T, need["mix"], dtype=dt, device=dev),
             act=torch.zeros(T, need["act"], dtype=dt, device=dev), y=torch.zeros(T, c.width, dtype=f32, device=dev),
