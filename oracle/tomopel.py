@@ -137,13 +137,17 @@ def relu2_ff(X, w_up, w_down):
     return torch.relu(X @ w_up.T).pow(2) @ w_down.T
 
 
-def routed_ff(X, w_router, correction, experts, top: int, shared=None):
+def routed_ff(X, w_router, correction, experts, top: int, shared=None, margins=None):
     """softmax scores over all experts; the `top` largest of score + correction are chosen; weights = the chosen scores
-    (without the correction) over their sum; experts = [(w_up, w_down)], each W_down relu(W_up h)^2"""
+    (without the correction) over their sum; experts = [(w_up, w_down)], each W_down relu(W_up h)^2.  margins (a list)
+    collects, per token, how far the last chosen expert's choice score stands above the first one left out."""
     s = torch.softmax(X @ w_router.T, -1)
     out = torch.zeros(X.shape[0], experts[0][1].shape[0], dtype=X.dtype)
     for t in range(X.shape[0]):
-        order = sorted(range(len(experts)), key=lambda e: (-float(s[t, e] + correction[e]), e))[:top]
+        ranked = sorted(range(len(experts)), key=lambda e: (-float(s[t, e] + correction[e]), e))
+        order = ranked[:top]
+        if margins is not None and top < len(experts):
+            margins.append(float(s[t, ranked[top - 1]] + correction[ranked[top - 1]] - s[t, ranked[top]] - correction[ranked[top]]))
         tot = sum(s[t, e] for e in order) + 1e-20
         for e in order:
             out[t] += (s[t, e] / tot) * relu2_ff(X[t:t + 1], *experts[e])[0]
@@ -160,7 +164,7 @@ class State:
         self.pos, self.layers = 0, {}
 
 
-def forward(cfg: dict, sd: dict, tokens, state: State | None = None, dtype=F, per_layer: bool = False):
+def forward(cfg: dict, sd: dict, tokens, state: State | None = None, dtype=F, per_layer: bool = False, margins=None):
     """tokens continue the sequence that `state` describes (None: a new one).  Returns logits [n, vocab] (and, with
     per_layer, the sum of the residual streams after every layer [L, n, W])."""
     w = {k: v.to(dtype) for k, v in sd.items()}
@@ -172,6 +176,8 @@ def forward(cfg: dict, sd: dict, tokens, state: State | None = None, dtype=F, pe
 
     def sublayer(xs, p, q, fn):
         hc = f"{p}hc{q}."
+        if hc + "in" not in w:                                        # no stream weights: the plain residual x + m f(norm(x))
+            return xs + m * fn(offset_rms_norm(xs.sum(0), w[f"{p}norm{q}"], eps))[None]
         h = offset_rms_norm(streams_read(xs, w[hc + "in"]), w[f"{p}norm{q}"], eps)
         return streams_write(xs, fn(h), w[hc + "mix"], w[hc + "out"], m)
 
@@ -185,15 +191,16 @@ def forward(cfg: dict, sd: dict, tokens, state: State | None = None, dtype=F, pe
                 return out
             a, b, past = mx["left"], mx["right"], st.layers.get(i, (None, None))
             pl, pr = p + "mix.left.", p + "mix.right."
+            qt = a.get("q_temp") or {"coef": 0.0, "every": 1}
             left, kv = biased_attention(h, w[pl + "q"], w[pl + "k"], w[pl + "v"], w[pl + "g"], w[pl + "o"], w[pl + "q.norm"],
-                                        w[pl + "k.norm"], w[pl + "rel"], H=a["heads"], G=a["kv_heads"], D=a["dim"], E=a["vdim"],
-                                        scale=a["scale"], far=a["bias_max"], temp_coef=a["q_temp"]["coef"],
-                                        temp_every=a["q_temp"]["every"], eps=eps, pos0=st.pos, past=past[0])
+                                        w[pl + "k.norm"], w[pl + "rel"], H=a["heads"], G=a.get("kv_heads", a["heads"]), D=a["dim"],
+                                        E=a.get("vdim", a["dim"]), scale=a["scale"], far=a["bias_max"], temp_coef=qt["coef"],
+                                        temp_every=qt["every"], eps=eps, pos0=st.pos, past=past[0])
             right, ss = ssd(h, w[pr + "in"], w[pr + "conv"], w[pr + "conv.b"], w[pr + "dt_bias"], w[pr + "A_log"], w[pr + "D"],
-                            w[pr + "norm"], w[pr + "o"], heads=b["heads"], vdim=b["vdim"], state=b["state"], groups=b["groups"],
-                            norm_groups=b["norm_groups"], eps=eps, past=past[1])
+                            w[pr + "norm"], w[pr + "o"], heads=b["heads"], vdim=b["vdim"], state=b["state"],
+                            groups=b.get("groups", 1), norm_groups=b.get("norm_groups", 1), eps=eps, past=past[1])
             st.layers[i] = (kv, ss)
-            return mx["left_scale"] * left + mx["right_scale"] * right
+            return mx.get("left_scale", 1.0) * left + mx.get("right_scale", 1.0) * right
 
         xs = sublayer(xs, p, 1, mixer)
         f = ly.get("mlp")
@@ -203,8 +210,8 @@ def forward(cfg: dict, sd: dict, tokens, state: State | None = None, dtype=F, pe
             else:
                 ex = [(w[p + f"mlp.e{e}.up"], w[p + f"mlp.e{e}.down"]) for e in range(f["router"]["experts"])]
                 sh = (w[p + "mlp.shared.up"], w[p + "mlp.shared.down"]) if f.get("shared") else None
-                xs = sublayer(xs, p, 2, lambda h: routed_ff(h, w[p + "mlp.router"], w[p + "mlp.correction"], ex,
-                                                            f["router"]["top"], sh))
+                corr = w.get(p + "mlp.correction", torch.zeros(len(ex), dtype=dtype))
+                xs = sublayer(xs, p, 2, lambda h: routed_ff(h, w[p + "mlp.router"], corr, ex, f["router"]["top"], sh, margins))
         trace.append(xs.sum(0))
     st.pos += len(tokens)
     logits = offset_rms_norm(xs.sum(0), w["final.norm"], eps) @ w["head"].T

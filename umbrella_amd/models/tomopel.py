@@ -91,7 +91,7 @@ def bias_by_distance(rel: torch.Tensor, far: float, max_len: int) -> torch.Tenso
     """the learned table [rows, heads] -> fp32 [heads, n_dist] indexed by the distance itself; distances from n_dist - 1 on
     share the last entry (every distance the table tells apart, or every distance a sequence of max_len can hold)"""
     rows = rel.shape[0]
-    n = int(max(1, min(max_len, math.ceil(far) + 1 if far > 0 else 1)))
+    n = int(max(1, min(max_len, max(math.ceil(far), rows // 2) + 1)))
     b = distance_buckets(rows, far, n)
     last = int((b == rows - 1).nonzero()[0]) if bool((b == rows - 1).any()) else n - 1
     return rel.to(torch.float32)[b[:last + 1].to(rel.device)].t().contiguous()
