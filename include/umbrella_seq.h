@@ -199,9 +199,13 @@ int umb_hc_read(float* u_out, void* h, const float* x, const int* rows, const fl
 /* ---- minimal gated recurrence, element by element over `Wm` channels: with the projections zr / ur / gr (fp32, biases
  * added, columns z_col / u_col / g_col of proj [T][ld]), z = sigmoid(zr), candidate = ur + 1/2 where ur >= 0, else
  * sigmoid(ur); S_t = (1 - z) S_(t-1) + z candidate; out[t] = S_t * silu(gr) in `dtype`.  state fp32 [slots][Wm]; a
- * sequence that starts at position 0 starts from S = 0 whatever its slot holds. */
+ * sequence that starts at position 0 starts from S = 0 whatever its slot holds.  max_len: the longest stretch of the step;
+ * long stretches run as pieces side by side (piece summaries, then a fold) when scratch (fp32, at least
+ * umb_mingru_scratch_floats(T, B, Wm) floats; no stream argument) is given, else token by token. */
+long umb_mingru_scratch_floats(int T, int B, int Wm);
 int umb_mingru_scan(void* out, float* state, const float* proj, int ld, int z_col, int u_col, int g_col, const int* seq_slot,
-                    const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int Wm, int dtype, umb_stream_t stream);
+                    const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int Wm, int max_len, float* scratch,
+                    long scratch_floats, int dtype, umb_stream_t stream);
 
 /* ---- linear recurrence with a matrix state per head, general operand placement (umb_gla_scan is one case of it):
  * S <- a_t S + k_t v_t^T, o_t = S^T (q_t * qscale); q and k rows [T][ldq / ldk] hold qk_heads groups of D (head h reads

@@ -8,6 +8,12 @@ synthetic ids.
         layers -- the closest existing model: same runtime, cache manager and engine -- at equal width, heads, window,
         feed-forward width and layer count
 
+    python bench.py --family tomopel [--sizes 1b,8b] ...
+        Tomopel (two residual streams; softmax attention with a distance bias beside a state-space layer; minGRU layers; dense
+        and routed relu^2 feed-forwards) beside Gitopel -- the closest existing model: grouped-query attention layers where
+        Tomopel has its parallel mixer, gated-linear-attention layers (the same scan kernel) where it has a minGRU -- at
+        equal width, heads x head size, feed-forward width and layer count
+
 or directly: python scripts/bench_seqmix.py.  One JSON line: per size, ms and tokens/s of
   prefill   one prompt of --prompt-len tokens in one step (Llama: its chunked prompt path)
   decode    one token per step behind that prompt, batch 1 (both) and batch --batch (Gitopel; the Llama runtime is batch 1)
@@ -45,6 +51,38 @@ FID_SIZES = {
 }
 
 
+# Tomopel: attention heads x dim (values vdim) over kv_heads, beside a state-space layer of s_heads x s_vdim with `state`
+# features per head; "p" layers have the parallel mixer, "g" layers a minGRU of the model's width; feed-forwards alternate
+# dense (ff) and experts (each ff / 4 wide, two of eight used, plus a shared one)
+TOM_SIZES = {
+    "1b": dict(width=2048, ff=8192, heads=32, kv_heads=8, dim=64, vdim=64, s_heads=32, s_vdim=64, state=128, groups=8, conv=4,
+               experts=8, top=2, pattern="pgpp", vocab=32000, bias_rows=32, bias_max=2048),
+    "8b": dict(width=4096, ff=14336, heads=32, kv_heads=8, dim=128, vdim=128, s_heads=64, s_vdim=64, state=128, groups=8, conv=4,
+               experts=8, top=2, pattern="pg", vocab=32000, bias_rows=32, bias_max=2048),
+}
+
+
+def tomopel_config(s):
+    layers = []
+    for i, ch in enumerate(s["pattern"]):
+        if ch == "p":
+            mixer = {"left": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["vdim"],
+                              "scale": s["dim"] ** -0.5, "bias_max": s["bias_max"], "q_temp": {"coef": 0.1, "every": 256}},
+                     "right": {"heads": s["s_heads"], "vdim": s["s_vdim"], "state": s["state"], "groups": s["groups"],
+                               "norm_groups": s["groups"], "conv": s["conv"]}, "left_scale": 1.0, "right_scale": 1.0}
+            kind = "parallel"
+        else:
+            mixer, kind = {"width": s["width"]}, "mingru"
+        if i % 2 == 0:
+            mlp = {"kind": "dense", "ff": s["ff"]}
+        else:
+            mlp = {"kind": "moe", "router": {"experts": s["experts"], "top": s["top"]}, "expert": {"ff": s["ff"] // 4},
+                   "shared": {"ff": s["ff"] // 4}}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Tomopel", "layers": layers, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0}, "streams": 2,
+            "residual_mult": 0.5, "vocab": s["vocab"], "width": s["width"]}
+
+
 def fidizen_config(s):
     mixer = {"heads": s["heads"], "dim": s["dim"], "rot_dim": s["rot"], "vdim": s["vdim"], "q_rank": s["q_rank"],
              "kv_rank": s["kv_rank"], "mask": {"size": s["window"]}, "rot": {"dims": s["rot"], "base": 10000.0},
@@ -75,15 +113,18 @@ def gitopel_config(s):
     return {"architecture": "Gitopel", "layers": layers, "norm": {"eps": 1e-6, "groups": 4}, "vocab": s["vocab"], "width": s["width"]}
 
 
-def device_state(cfg, dtype, seed=0, rank=16, shapes=None):
+def device_state(cfg, dtype, seed=0, rank=16, shapes=None, zero_norms=False):
     """random checkpoint drawn on the device in the storage dtype"""
     from umbrella_amd.models import gitopel
     g = torch.Generator(device="cuda").manual_seed(seed)
     sd = {}
     for name, shape in (shapes or gitopel.tensor_shapes(cfg, rank)).items():
         leaf = name.split(".")[-1]
-        if "norm" in leaf:
-            sd[name] = torch.ones(shape, dtype=dtype, device="cuda")
+        if ".hc" in name:                               # stream tables near the plain residual
+            base = torch.eye(shape[0]) if len(shape) == 2 else torch.full(shape, 1.0 if leaf == "out" else 1.0 / shape[0])
+            sd[name] = (base.cuda() + 0.05 * torch.randn(shape, generator=g, device="cuda")).to(dtype)
+        elif "norm" in leaf:
+            sd[name] = torch.full(shape, 0.0 if zero_norms and "mix." not in name else 1.0, dtype=dtype, device="cuda")
         elif len(shape) == 1:
             sd[name] = (0.1 * torch.randn(shape, generator=g, device="cuda")).to(dtype)
         else:
@@ -100,13 +141,18 @@ def timed(fn, reps):
     return (time.time() - t0) / reps * 1e3
 
 
-def bench_gitopel(s, args, dtype, fidizen=False):
+def bench_gitopel(s, args, dtype, fidizen=False, tomopel=False):
     from umbrella_amd.models import fidizen as fid
     from umbrella_amd.models import gitopel
+    from umbrella_amd.models import tomopel as tom
     B, P, steps = args.batch, args.prompt_len, args.decode_steps
     kw = dict(batch_size=B + 1, max_length=P + 2 * steps + 8, max_tokens=(B + 1) * (P + 2 * steps + 8), device="cuda:0",
               dtype=dtype, max_step_tokens=max(P, B))
-    if fidizen:
+    if tomopel:
+        cfg = tom.config_from_dict(tomopel_config(s))
+        sd = device_state(cfg, dtype, shapes=tom.tensor_shapes(cfg, s["bias_rows"]), zero_norms=True)
+        m = tom.Tomopel("bench", state_dict=sd, config=cfg, **kw)
+    elif fidizen:
         cfg = fid.config_from_dict(fidizen_config(s))
         m = fid.Fidizen("bench", state_dict=device_state(cfg, dtype, shapes=fid.tensor_shapes(cfg)), config=cfg, **kw)
     else:
@@ -192,6 +238,31 @@ def run_fidizen(args):
     return line
 
 
+def run_tomopel(args):
+    """Tomopel beside Gitopel at equal width, heads x head size, feed-forward width and layer count: attention layers for the
+    parallel mixers, gated-linear-attention layers for the minGRU layers"""
+    import __graft_entry__ as ge
+    ge.build_seq()
+    dtype = torch.bfloat16
+    res = {}
+    for name in args.sizes.split(","):
+        s = TOM_SIZES[name]
+        res[name] = {"shape": dict(s)}
+        res[name]["tomopel"] = bench_gitopel(s, args, dtype, tomopel=True)
+        torch.cuda.empty_cache()
+        if not args.no_gitopel:
+            g = dict(width=s["width"], ff=s["ff"], heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], gheads=s["s_heads"] // 4,
+                     gdim=s["state"], gvdim=4 * s["s_vdim"], window=args.prompt_len + 2 * args.decode_steps + 8, pool=16,
+                     pattern=s["pattern"].replace("p", "a"), vocab=s["vocab"])
+            res[name]["gitopel_equal_size"] = bench_gitopel(g, args, dtype)
+            torch.cuda.empty_cache()
+    line = {"metric": "prefill / decode throughput, Tomopel beside Gitopel at equal size", "unit": "tokens/s",
+            "dtype": "bf16", "data": "synthetic: random weights, random ids", "n_gpus": 1, "prompt_len": args.prompt_len,
+            "decode_steps": args.decode_steps, "batch": args.batch, "sizes": res}
+    print(json.dumps(line), flush=True)
+    return line
+
+
 def run(args):
     import __graft_entry__ as ge
     ge.build()
@@ -224,7 +295,7 @@ def add_args(ap):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--prompt-len", type=int, default=2048)
-    ap.add_argument("--family", default="gitopel", choices=["gitopel", "fidizen"])
+    ap.add_argument("--family", default="gitopel", choices=["gitopel", "fidizen", "tomopel"])
     add_args(ap)
     a = ap.parse_args()
-    run_fidizen(a) if a.family == "fidizen" else run(a)
+    {"fidizen": run_fidizen, "tomopel": run_tomopel}.get(a.family, run)(a)

@@ -128,7 +128,8 @@ def test_stream_seam_with_trivial_tables_is_the_plain_residual(lib):
 
 # ------------------------------------------------------------------ minimal gated recurrence
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("Wm,splits", [(24, [19]), (70, [1] * 12), (300, [2, 9, 1, 1, 17, 3]), (257, [40, 1, 1])])
+@pytest.mark.parametrize("Wm,splits", [(24, [19]), (70, [1] * 12), (300, [2, 9, 1, 1, 17, 3]), (257, [40, 1, 1]),
+                                       (70, [333]), (24, [129, 1, 200, 2, 131]), (300, [128, 160])])      # long stretches: pieces
 def test_mingru_scan_prompt_portions_and_single_tokens(lib, dtype, Wm, splits):
     """the state is carried across steps; a second sequence in the batch with other lengths does not disturb it; the slot's old
     state is ignored by a sequence that starts at position 0"""
@@ -152,8 +153,10 @@ def test_mingru_scan_prompt_portions_and_single_tokens(lib, dtype, Wm, splits):
         both = torch.cat([proj2[at2:at2 + c2], proj[at:at + cnt]])
         st = Steps([c2, cnt], [at2, at], [0, 2])
         out = torch.zeros(st.T, Wm, dtype=dtype, device="cuda:0")
+        need = _lib.load_seq().umb_mingru_scratch_floats(st.T, 2, Wm)
+        scratch = torch.zeros(need, dtype=torch.float32, device="cuda:0")
         _lib.seq_call("umb_mingru_scan", out, state, dev(both), both.shape[1], 2, 2 + Wm, 2 + 2 * Wm, st.d["seq_slot"],
-                      st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 2, Wm, code(dtype))
+                      st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 2, Wm, max(c2, cnt), scratch, need, code(dtype))
         got2.append(out[:c2].clone())
         got.append(out[c2:].clone())
         at, at2 = at + cnt, at2 + c2
@@ -289,9 +292,13 @@ def _run_attn(lib, X, w, dtype, splits, H, G, D, E, scale, far, temp, eps, page=
         out = torch.zeros(cnt, H * E + 3, dtype=dtype, device="cuda:0")
         _lib.seq_call("umb_bsa_prep", q, kv, proj, ld, dev(w["q_norm"], dtype), dev(w["k_norm"], dtype), st.d["pos"], st.d["slot"], cnt,
                       H, G, D, E, temp[0], temp[1], eps, code(dtype))
-        _lib.seq_call("umb_bsa_attend", out, H * E + 3, q, kv, proj, ld, H * D + G * D + G * E, bias,
-                      bias.shape[1] if bias is not None else 0, st.d["pos"], st.d["slot"], cnt, H, G, D, E, window, scale, out_scale,
-                      code(dtype))
+        nd = bias.shape[1] if bias is not None else 0
+        if cnt >= 16 and lib.umb_bsa_attend_tiled_ok(H, G, D, E, code(dtype)):       # as the forward chooses: the matrix pipe
+            _lib.seq_call("umb_bsa_attend_tiled", out, H * E + 3, q, kv, proj, ld, H * D + G * D + G * E, bias, nd, st.d["seq_slot"],
+                          st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, cnt, H, G, D, E, window, scale, out_scale, code(dtype))
+        else:
+            _lib.seq_call("umb_bsa_attend", out, H * E + 3, q, kv, proj, ld, H * D + G * D + G * E, bias, nd, st.d["pos"],
+                          st.d["slot"], cnt, H, G, D, E, window, scale, out_scale, code(dtype))
         assert float(out[:, H * E:].abs().max()) == 0.0
         outs.append(out[:, :H * E].clone())
         at += cnt
@@ -310,6 +317,7 @@ def _attn_oracle(X, w, dtype, H, G, D, E, scale, far, temp, eps):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,E,rows,far,temp", [(4, 2, 8, 6, 12, 40, (0.3, 8)), (3, 1, 7, 9, 4, 9, (0.0, 0)), (2, 2, 16, 16, 7, 25, (0.5, 1)),
                                                    (8, 2, 32, 64, 32, 70, (0.2, 16)), (6, 3, 24, 130, 9, 1000, (0.1, 5)),
+                                                   (12, 1, 40, 48, 10, 33, (0.2, 7)), (4, 4, 136, 144, 6, 20, (0.0, 0)),
                                                    (1, 1, 8, 200, 16, 16, (1.0, 64))])
 def test_biased_attention_prompt_portions_and_single_tokens(lib, dtype, H, G, D, E, rows, far, temp):
     """every bucket of the table is reached (far < n for most shapes), the temperature steps several times, keys sit on both

@@ -294,7 +294,8 @@ SEQ_SIGNATURES = {
     "umb_hc_embed": [_P, _P, _P, _P, _F, _P, _P, _F, _I, _I, _I, _I, _F, _I],
     "umb_hc_seam": [_P, _P, _P, _P, _P, _F, _P, _P, _F, _I, _I, _I, _F, _I],
     "umb_hc_read": [_P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _F, _I],
-    "umb_mingru_scan": [_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I],
+    "umb_mingru_scratch_floats": [_I, _I, _I],
+    "umb_mingru_scan": [_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _P, _L, _I],
     "umb_lin_scan": [_P, _P, _P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _F],
     "umb_ssd_prep": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
     "umb_ssd_conv_update": [_P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
@@ -310,7 +311,7 @@ SEQ_SIGNATURES = {
     "umb_sample_rows": [_P, _P, _I, _I, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P],
     "umb_seq_version": [],
 }
-_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok", "umb_seq_resid_canon_step_ok", "umb_bsa_attend_tiled_ok"}          # predicates: no stream argument, the value is the answer
+_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok", "umb_seq_resid_canon_step_ok", "umb_bsa_attend_tiled_ok", "umb_mingru_scratch_floats"}          # predicates: no stream argument, the value is the answer
 _seq_lib = None
 
 
@@ -329,7 +330,7 @@ def load_seq() -> C.CDLL:
         if name == "umb_seq_version":
             fn.argtypes, fn.restype = [], C.c_char_p
         elif name in _SEQ_NO_STREAM:
-            fn.argtypes, fn.restype = list(args), C.c_int
+            fn.argtypes, fn.restype = list(args), (C.c_long if name.endswith("_floats") else C.c_int)
         else:
             fn.argtypes, fn.restype = list(args) + [_P], C.c_int
     _seq_lib = lib

@@ -253,18 +253,267 @@ extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPaged
   return UMB_OK;
 }
 
-// the matrix-pipe prompt kernel is declared in the header; until a shape is covered the forward takes the kernel above
+// ---- prompt attention on the matrix pipe (16-bit storage; D a multiple of 8, E a multiple of 16).
+// Workgroup = (16 consecutive positions of one sequence, one key/value head, a block of 4 HPW of its query heads); wave w owns
+// HPW heads.  The tile's keys -- from the first position's window start to the last position -- are walked in steps of 32 by
+// the whole workgroup: the step's 32 cached key rows and value rows are staged ONCE into LDS (keys as cached: the A operand of
+// S^T = K Q^T; values transposed: the A operand of O^T += V^T P^T) and serve every head of the workgroup; the next step's rows
+// are in flight in registers while the current one is used.  Per step and head: two 16-key score tiles; the bias of the
+// lane's eight (query, key) pairs, fetched by distance before the products are issued; online softmax in fp32 with base-2
+// exponents, accumulators rescaled only when a maximum moved; the lane's eight weights ARE its share of the B operand of the
+// value product.  Scores and weights keep fp32 accuracy on the 16-bit pipe: the fp32 queries and the fp32 weights enter as
+// high + low 16-bit halves (two products each, 2^-17 relative).
+constexpr float BSA_LOG2E = 1.4426950408889634f;
+
+template <typename P> __device__ __forceinline__ void split2(float a, float b, unsigned& hi, unsigned& lo) {
+  const u16 ah = P::from_f(a), bh = P::from_f(b);
+  hi = (unsigned)ah | ((unsigned)bh << 16);
+  lo = pack2<P>(a - P::to_f(ah), b - P::to_f(bh));
+}
+
+template <typename P, int NSM, int NVM, int HPW>
+__global__ __launch_bounds__(256) void bsa_attend_mfma_kernel(u16* __restrict__ out, int ldo, const float* __restrict__ q,
+                                                              UmbPagedKV kv, const float* __restrict__ proj, int ld, int gate_col,
+                                                              const float* __restrict__ bias, int n_dist,
+                                                              const int* __restrict__ seq_slot, const int* __restrict__ seq_row0,
+                                                              const int* __restrict__ seq_pos0, const int* __restrict__ seq_len,
+                                                              int H, int G, int D, int E, int window, float scale, float out_scale) {
+  extern __shared__ __attribute__((aligned(16))) u16 bsa_lds[];
+  constexpr int NLK = (NSM * 4 + 7) / 8, NLV = (NVM * 2 + 7) / 8;     // 16-byte chunks of a key / value row per staging thread
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g4 = lane >> 4;
+  const int LD = D + 8;                               // LDS row stride of the key tile: 16 bytes of padding spread the banks
+  const int ns = (D + 31) >> 5, nv = E >> 4, nck = D >> 3, ncv = E >> 3;
+  constexpr int LT = 36;                              // row stride of the transposed value tile: 32 keys + 8 bytes of padding
+  u16* k_s = bsa_lds;                                 // [32][LD]
+  u16* v_t = bsa_lds + 32 * LD;                       // [E][LT]
+  const int b = blockIdx.y;
+  const int n = seq_len[b], q0 = blockIdx.x * 16;
+  if (q0 >= n) return;                                // the whole workgroup
+  const int hpg = H / G, hblocks = (hpg + 4 * HPW - 1) / (4 * HPW);
+  const int g = blockIdx.z / hblocks;
+  const int hl0 = ((blockIdx.z % hblocks) * 4 + wave) * HPW;         // first of the wave's heads inside the group
+  const bool active = hl0 < hpg;                      // a wave without heads still stages rows and meets the barriers
+  const int slot = seq_slot[b], row0 = seq_row0[b], pos0 = seq_pos0[b];
+  const int nq = n - q0 < 16 ? n - q0 : 16;
+  const int i_first = pos0 + q0, i_last = i_first + nq - 1;
+  const bool q_ok = j < nq;
+  const int i_j = i_first + (q_ok ? j : nq - 1);
+  const long qrow = row0 + q0 + (q_ok ? j : nq - 1);
+  const int j_lo = i_first - window + 1 > 0 ? i_first - window + 1 : 0;
+  const int total = i_last - j_lo + 1;
+  const float scale2 = scale * BSA_LOG2E;
+  const u16* kbase = reinterpret_cast<const u16*>(kv.k);
+  const u16* vbase = reinterpret_cast<const u16*>(kv.v);
+  u32x4 qh[HPW][NSM], ql[HPW][NSM];
+  f32x4 o[HPW][NVM];
+  float m_run[HPW], l_run[HPW];
+  bool h_ok[HPW];
+  int hd[HPW];
+#pragma unroll
+  for (int hh = 0; hh < HPW; ++hh) {
+    h_ok[hh] = hl0 + hh < hpg;
+    hd[hh] = g * hpg + (h_ok[hh] ? hl0 + hh : hpg - 1);
+    const float* qr = q + (qrow * H + hd[hh]) * D;
+#pragma unroll
+    for (int s = 0; s < NSM; ++s) {
+      const int d = 32 * s + 8 * g4;
+      qh[hh][s] = u32x4{0u, 0u, 0u, 0u};
+      ql[hh][s] = u32x4{0u, 0u, 0u, 0u};
+      if (s < ns && d < D) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(qr + d), c = *reinterpret_cast<const f32x4*>(qr + d + 4);
+        unsigned hi[4], lo[4];
+        split2<P>(a[0], a[1], hi[0], lo[0]);
+        split2<P>(a[2], a[3], hi[1], lo[1]);
+        split2<P>(c[0], c[1], hi[2], lo[2]);
+        split2<P>(c[2], c[3], hi[3], lo[3]);
+        qh[hh][s] = u32x4{hi[0], hi[1], hi[2], hi[3]};
+        ql[hh][s] = u32x4{lo[0], lo[1], lo[2], lo[3]};
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < NVM; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run[hh] = -INFINITY;
+    l_run[hh] = 0.f;
+  }
+  // staging role of a thread: key row sm of the step, 16-byte chunks sc, sc + 8, ... of that row (keys and values)
+  const int sm = threadIdx.x & 31, sc = threadIdx.x >> 5;
+  u32x4 stk[NLK], stv[NLV];
+  auto fetch = [&](int base) {
+    const int kx = base + sm;
+    const bool ok = kx < total;
+    const long offk = ok ? pkv_tok(kv, slot, j_lo + kx, g, G, D) : 0;
+    const long offv = ok ? pkv_tok(kv, slot, j_lo + kx, g, G, E) : 0;
+#pragma unroll
+    for (int u = 0; u < NLK; ++u) {
+      const int ch = sc + 8 * u;
+      stk[u] = (ok && ch < nck) ? *reinterpret_cast<const u32x4*>(kbase + offk + 8 * ch) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < NLV; ++u) {
+      const int ch = sc + 8 * u;
+      stv[u] = (ok && ch < ncv) ? *reinterpret_cast<const u32x4*>(vbase + offv + 8 * ch) : u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  fetch(0);
+  for (int base = 0; base < total; base += 32) {
+    __syncthreads();                                  // every wave is done with the previous tile
+#pragma unroll
+    for (int u = 0; u < NLK; ++u) {
+      const int ch = sc + 8 * u;
+      if (ch < nck) *reinterpret_cast<u32x4*>(k_s + sm * LD + 8 * ch) = stk[u];
+    }
+#pragma unroll
+    for (int u = 0; u < NLV; ++u) {
+      const int ch = sc + 8 * u;
+      if (ch < ncv) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v_t[(8 * ch + 2 * e) * LT + sm] = (u16)(stv[u][e] & 0xffffu);
+          v_t[(8 * ch + 2 * e + 1) * LT + sm] = (u16)(stv[u][e] >> 16);
+        }
+      }
+    }
+    __syncthreads();
+    if (base + 32 < total) fetch(base + 32);          // in flight while this step is used
+    if (!active) continue;
+    // which of the lane's eight keys this query sees, and at what distance: the same for every head
+    bool vis[8];
+    int di[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int jt = j_lo + base + 16 * (e >> 2) + 4 * g4 + (e & 3);
+      vis[e] = q_ok && jt <= i_j && jt > i_j - window;
+      const int dd = i_j - jt;
+      di[e] = dd < 0 ? 0 : (dd < n_dist ? dd : n_dist - 1);
+    }
+    float bv[HPW][8];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bv[hh][e] = bias ? bias[(long)hd[hh] * n_dist + di[e]] : 0.f;
+    f32x4 sc2[HPW][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int hh = 0; hh < HPW; ++hh) sc2[hh][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const u16* kr = k_s + (16 * u + j) * LD;
+#pragma unroll
+      for (int s = 0; s < NSM; ++s) {
+        const int d = 32 * s + 8 * g4;
+        if (s < ns) {
+          const u32x4 kf = d < D ? *reinterpret_cast<const u32x4*>(kr + d) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+          for (int hh = 0; hh < HPW; ++hh) {
+            sc2[hh][u] = P::mfma(kf, ql[hh][s], sc2[hh][u]);
+            sc2[hh][u] = P::mfma(kf, qh[hh][s], sc2[hh][u]);
+          }
+        }
+      }
+    }
+    u32x4 ph[HPW], pl[HPW];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      // maxima and exponents in base 2 (scale2 = scale log2 e): one v_exp_f32 per weight
+      float sv[8], mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        sv[e] = vis[e] ? sc2[hh][e >> 2][e & 3] * scale2 + bv[hh][e] * BSA_LOG2E : -INFINITY;
+        mx = fmaxf(mx, sv[e]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[hh], mx);
+      const float m_ref = m_new == -INFINITY ? 0.f : m_new;          // a row that has seen no key yet: all weights 0
+      const float fac = __builtin_amdgcn_exp2f(m_run[hh] - m_ref);
+      float w[8], sum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        w[e] = __builtin_amdgcn_exp2f(sv[e] - m_ref);
+        sum += w[e];
+      }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l_run[hh] = l_run[hh] * fac + sum;
+      m_run[hh] = m_new;
+      if (__ballot(fac != 1.f)) {                                    // the maximum moved for some row of the tile
+#pragma unroll
+        for (int dt = 0; dt < NVM; ++dt) {
+          if (dt < nv) { o[hh][dt][0] *= fac; o[hh][dt][1] *= fac; o[hh][dt][2] *= fac; o[hh][dt][3] *= fac; }
+        }
+      }
+      unsigned hi[4], lo[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) split2<P>(w[2 * e], w[2 * e + 1], hi[e], lo[e]);
+      ph[hh] = u32x4{hi[0], hi[1], hi[2], hi[3]};
+      pl[hh] = u32x4{lo[0], lo[1], lo[2], lo[3]};
+    }
+    // O^T[d][query] += V^T[d][keys] P^T[keys][query]: lane (d row j of tile dt, quad g4) reads its 8 keys' values
+#pragma unroll
+    for (int dt = 0; dt < NVM; ++dt) {
+      if (dt < nv) {
+        const u16* vr = v_t + (16 * dt + j) * LT + 4 * g4;
+        const u32x2 t0 = *reinterpret_cast<const u32x2*>(vr), t1 = *reinterpret_cast<const u32x2*>(vr + 16);
+        const u32x4 va = u32x4{t0[0], t0[1], t1[0], t1[1]};
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+          o[hh][dt] = P::mfma(va, pl[hh], o[hh][dt]);
+          o[hh][dt] = P::mfma(va, ph[hh], o[hh][dt]);
+        }
+      }
+    }
+  }
+  // lane holds O^T[d = 16 dt + 4 g4 + rr][query j]
+  if (q_ok && active) {
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      if (!h_ok[hh]) continue;
+      const float gt = gate_col >= 0 ? 1.f / (1.f + expf(-proj[qrow * ld + gate_col + hd[hh]])) : 1.f;
+      const float inv = out_scale * gt / l_run[hh];
+      u16* orow = out + qrow * ldo + (long)hd[hh] * E;
+#pragma unroll
+      for (int dt = 0; dt < NVM; ++dt) {
+        if (dt < nv) {
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) orow[16 * dt + 4 * g4 + rr] = P::from_f(o[hh][dt][rr] * inv);
+        }
+      }
+    }
+  }
+}
+
 extern "C" int umb_bsa_attend_tiled_ok(int H, int G, int D, int E, int dtype) {
-  (void)H; (void)G; (void)D; (void)E; (void)dtype;
-  return 0;
+  return H >= 1 && G >= 1 && H % G == 0 && (dtype == UMB_SEQ_BF16 || dtype == UMB_SEQ_F16) && D >= 8 && D % 8 == 0 && D <= 256 &&
+         E >= 16 && E % 16 == 0 && E <= 256;
 }
 
 extern "C" int umb_bsa_attend_tiled(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld,
                                     int gate_col, const float* bias, int n_dist, const int* seq_slot, const int* seq_row0,
                                     const int* seq_pos0, const int* seq_len, int B, int max_len, int H, int G, int D, int E,
                                     int window, float scale, float out_scale, int dtype, hipStream_t st) {
-  (void)out; (void)ldo; (void)q; (void)kv; (void)proj; (void)ld; (void)gate_col; (void)bias; (void)n_dist; (void)seq_slot;
-  (void)seq_row0; (void)seq_pos0; (void)seq_len; (void)B; (void)max_len; (void)H; (void)G; (void)D; (void)E; (void)window;
-  (void)scale; (void)out_scale; (void)dtype; (void)st;
-  return UMB_EINVAL;
+  if (B < 1 || B > 65535 || max_len < 1 || window < 1 || !out || !q || !bsa_kv_ok(kv) || !seq_slot || !seq_row0 || !seq_pos0 ||
+      !seq_len || ldo < H * E || (bias && n_dist < 1) || (gate_col >= 0 && (!proj || ld < gate_col + H)) ||
+      !umb_bsa_attend_tiled_ok(H, G, D, E, dtype))
+    return UMB_EINVAL;
+  if (!bias) n_dist = 1;
+  const int hpg = H / G;
+  const size_t lds = ((size_t)32 * (D + 8) + (size_t)E * 36) * sizeof(u16);
+#define BSA_MFMA(NSM, NVM, HPW)                                                                                            \
+  do {                                                                                                                     \
+    const int hblocks = (hpg + 4 * HPW - 1) / (4 * HPW);                                                                   \
+    if ((long)G * hblocks > 65535) return UMB_EINVAL;                                                                      \
+    const dim3 grid((max_len + 15) / 16, B, G * hblocks);                                                                  \
+    if (ensure_dynamic_lds<bsa_attend_mfma_kernel<P, NSM, NVM, HPW>>(lds) != UMB_OK) return UMB_EHIP;                      \
+    hipLaunchKernelGGL((bsa_attend_mfma_kernel<P, NSM, NVM, HPW>), grid, dim3(256), lds, st, (u16*)out, ldo, q, *kv, proj, \
+                       ld, gate_col, bias, n_dist, seq_slot, seq_row0, seq_pos0, seq_len, H, G, D, E, window, scale,       \
+                       out_scale);                                                                                         \
+  } while (0)
+#define BSA_MFMA_SHAPE()                                                                                                   \
+  if (D <= 128 && E <= 128) { if (hpg > 4) BSA_MFMA(4, 8, 2); else BSA_MFMA(4, 8, 1); }                                    \
+  else BSA_MFMA(8, 16, 1)
+  if (dtype == UMB_SEQ_BF16) { using P = BF16; BSA_MFMA_SHAPE(); }
+  else { using P = F16; BSA_MFMA_SHAPE(); }
+#undef BSA_MFMA_SHAPE
+#undef BSA_MFMA
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
 }

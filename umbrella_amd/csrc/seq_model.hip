@@ -104,8 +104,9 @@ static int feed_forward(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
 static int mix_mingru(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSeqWork* ws, const UmbSeqStep* s, hipStream_t st) {
   const int Wm = ly.dim;
   if (ly.proj.N != 3 * Wm || !ly.state || ly.out.K != Wm) return UMB_EINVAL;
+  // ws->aux holds the piece summaries of long stretches (sized by the runtime: umb_mingru_scratch_floats of Tmax rows)
   return umb_mingru_scan(ws->mix, ly.state, ws->proj, 3 * Wm, 0, Wm, 2 * Wm, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B,
-                         Wm, m->dtype, st);
+                         Wm, s->max_len, ws->aux, umb_mingru_scratch_floats(s->T, s->B, Wm), m->dtype, st);
 }
 
 // softmax attention with a distance bias beside a state-space layer; both read the projection of the same input and write

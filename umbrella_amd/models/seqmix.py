@@ -250,7 +250,7 @@ class SeqMixLM(LLMBase):
                 ask(act=max(m.q_rank, m.heads * m.kv_rank), o=m.heads * (m.dim + m.rot_dim), mix=m.heads * max(m.dim, m.vdim),
                     aux=m.heads * (m.kv_rank + m.rot_dim))
             elif m.kind == "mingru":
-                ask(mix=m.dim)
+                ask(mix=m.dim, aux=3 * m.dim + m.dim // 16 + 1)     # aux: piece summaries and start states of long stretches
             elif m.kind == "attention_ssd":
                 # aux: queries | convolved [dt x | B | C | x] | decays; o: the scan's read-out; mix: [attention | state space]
                 inner = m.s_heads * m.s_vdim
