@@ -2,7 +2,9 @@
  *
  * Decoder stacks whose layers mix tokens with something other than the dense tree-masked softmax attention of
  * libumbrella_hip.so: gated linear attention (a per-head matrix state carried from token to token) and sliding-window
- * attention over a paged key/value store with mean-pooled blocks behind the window and sigmoid (un-normalised) weights.
+ * attention over a paged key/value store with mean-pooled blocks behind the window and sigmoid (un-normalised) weights;
+ * latent attention; a minimal gated recurrence; softmax attention with a bias by distance beside a state-space layer with a
+ * scalar decay per head; residuals of one or several streams; dense, PolyNorm and routed-expert feed-forwards.
  * The layer list, every size and every constant are data (UmbSeqLayer); one forward entry point walks the list.
  *
  * Conventions are those of umbrella_hip.h: extern "C", plain pointers and sizes, 0 or a negative errno-style code,
@@ -219,13 +221,14 @@ int umb_lin_scan(float* o, float* state, const float* q, int ldq, const float* k
  * [z (H Dv) | x (H Dv) | B (G N) | C (G N) | dt (H)].  prep: x, B, C through a causal convolution per channel (w [C][taps],
  * last column the token's own, bias b, inputs of earlier steps from conv_state fp32 [slots][taps - 1][C], the input of
  * position p in row p % (taps - 1)) and silu; dt = softplus(dt + dt_bias[h]); sx fp32 [T][lds] = [dt x | B | C | x],
- * alpha [T][H] = exp(-exp(a_log[h]) dt).  conv_update, launched after prep, stores the step's last raw inputs.
+ * alpha [T][H] = exp(-exp(a_log[h]) dt).  conv_update, launched after prep, stores the step's last raw inputs; with
+ * update_state (steps of ONE token per sequence only) prep stores the token's input itself and conv_update is not needed.
  * The recurrence itself is umb_lin_scan (k = B, v = dt x, q = C).
  * gate: y = o + d_skip[h] x, times silu(z), unit RMS in `norm_groups` equal parts of the H Dv row, times w, times
  * out_scale, in `dtype` at out[t ldo + ...]. */
 int umb_ssd_prep(float* sx, int lds, float* alpha, const float* proj, int ld, int col0, const void* conv_w, const void* conv_b,
-                 const float* conv_state, const float* dt_bias, const float* a_log, const int* pos, const int* slot, int T, int H,
-                 int Dv, int G, int N, int taps, int dtype, umb_stream_t stream);
+                 float* conv_state, const float* dt_bias, const float* a_log, const int* pos, const int* slot, int T, int H,
+                 int Dv, int G, int N, int taps, int update_state, int dtype, umb_stream_t stream);
 int umb_ssd_conv_update(float* conv_state, const float* proj, int ld, int col0, const int* seq_slot, const int* seq_row0,
                         const int* seq_pos0, const int* seq_len, int B, int C, int taps, umb_stream_t stream);
 int umb_ssd_gate(void* out, int ldo, const float* o, const float* sx, int lds, int x_col, const float* proj, int ld, int z_col,
@@ -238,13 +241,14 @@ int umb_ssd_gate(void* out, int ldo, const float* o, const float* sx, int lds, i
  * the heads; null: 1); cache K <- unit_rms(k) * w_k; cache V <- unit_rms(v) (no weight).
  * attend: score(i, j, h) = q_i . k_j * scale + bias[h][min(i - j, n_dist - 1)] over j <= i with i - j < window (bias fp32
  * [H][n_dist], null: none); softmax; out[t ldo + h E ..] = out_scale * sigmoid(gate[t][h]) * sum_j p_j v_j in `dtype`
- * (gate_col < 0: no gate). */
+ * (gate_col < 0: no gate).  scratch (fp32, may be null): with it, steps of few rows deal each row's keys to several workgroups
+ * (as many as T H 16 (E + 2) floats allow, at most 16) and merge the partial results in a second launch. */
 int umb_bsa_prep(float* q, const UmbPagedKV* kv, const float* proj, int ld, const void* w_q, const void* w_k, const int* pos,
                  const int* slot, int T, int H, int G, int D, int E, float temp_coef, int temp_every, float eps, int dtype,
                  umb_stream_t stream);
 int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
                    const float* bias, int n_dist, const int* pos, const int* slot, int T, int H, int G, int D, int E, int window,
-                   float scale, float out_scale, int dtype, umb_stream_t stream);
+                   float scale, float out_scale, float* scratch, long scratch_floats, int dtype, umb_stream_t stream);
 /* the same for steps that bring stretches of a sequence, on the matrix pipe (16-bit storage; umb_bsa_attend_tiled_ok says
  * 1 / 0 whether the kernel covers a shape and dtype; it has no stream): workgroups own 16 consecutive positions */
 int umb_bsa_attend_tiled_ok(int H, int G, int D, int E, int dtype);
@@ -350,6 +354,7 @@ typedef struct UmbSeqWork {
   void* moe_act;      /* [pairs][max expert_ff] dtype */
   float* moe_y;       /* [pairs][W] fp32 */
   int64_t moe_max_tiles;
+  int64_t aux_floats;  /* floats in aux (what a step does not use of it serves as scratch) */
 } UmbSeqWork;
 
 typedef struct UmbSeqStep {

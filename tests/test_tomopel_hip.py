@@ -191,10 +191,12 @@ def _run_ssd(lib, X, w, dtype, splits, H, Dv, N, G, NG, taps, eps, scale=1.0, sl
         alpha = torch.zeros(cnt, H, dtype=torch.float32, device="cuda:0")
         o = torch.zeros(cnt, inner, dtype=torch.float32, device="cuda:0")
         out = torch.zeros(cnt, inner + 2, dtype=dtype, device="cuda:0")
+        single = int(cnt == 1)                                          # as the forward does: one launch for single tokens
         _lib.seq_call("umb_ssd_prep", sx, lds + 1, alpha, proj, ld, col0, dev(w["conv_w"], dtype), dev(w["conv_b"], dtype), conv,
-                      f32("dt_bias"), f32("a_log"), st.d["pos"], st.d["slot"], cnt, H, Dv, G, N, taps, code(dtype))
-        _lib.seq_call("umb_ssd_conv_update", conv, proj, ld, col0 + inner, st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"],
-                      st.d["seq_len"], 1, C, taps)
+                      f32("dt_bias"), f32("a_log"), st.d["pos"], st.d["slot"], cnt, H, Dv, G, N, taps, single, code(dtype))
+        if not single:
+            _lib.seq_call("umb_ssd_conv_update", conv, proj, ld, col0 + inner, st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"],
+                          st.d["seq_len"], 1, C, taps)
         _lib.seq_call("umb_lin_scan", o, state, sx[:, inner + gn:], lds + 1, sx[:, inner:], lds + 1, sx, lds + 1, alpha, 1, G,
                       st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, H, N, Dv, 1.0)
         _lib.seq_call("umb_ssd_gate", out, inner + 2, o, sx, lds + 1, C, proj, ld, col0, f32("d_skip"), dev(w["norm_w"], dtype), cnt, H,
@@ -269,7 +271,7 @@ def _attn_weights(width, H, G, D, E, rows, seed):
 
 
 def _run_attn(lib, X, w, dtype, splits, H, G, D, E, scale, far, temp, eps, page=4, cache=None, seq="s", out_scale=1.0, window=2 ** 30,
-              max_len=512):
+              max_len=512, split_keys=True):
     """prep + attend through their entry points over a cache handed out by the cache manager -> [n, H E]"""
     from umbrella_amd import _lib
     from umbrella_amd.attn.cache import PagedSeqCache
@@ -297,8 +299,11 @@ def _run_attn(lib, X, w, dtype, splits, H, G, D, E, scale, far, temp, eps, page=
             _lib.seq_call("umb_bsa_attend_tiled", out, H * E + 3, q, kv, proj, ld, H * D + G * D + G * E, bias, nd, st.d["seq_slot"],
                           st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, cnt, H, G, D, E, window, scale, out_scale, code(dtype))
         else:
+            # steps of few rows with scratch: the keys of a row are dealt to several workgroups and merged
+            need = cnt * H * 16 * (E + 2) if split_keys else 0
+            scratch = torch.zeros(max(need, 1), dtype=torch.float32, device="cuda:0") if split_keys else None
             _lib.seq_call("umb_bsa_attend", out, H * E + 3, q, kv, proj, ld, H * D + G * D + G * E, bias, nd, st.d["pos"],
-                          st.d["slot"], cnt, H, G, D, E, window, scale, out_scale, code(dtype))
+                          st.d["slot"], cnt, H, G, D, E, window, scale, out_scale, scratch, need, code(dtype))
         assert float(out[:, H * E:].abs().max()) == 0.0
         outs.append(out[:, :H * E].clone())
         at += cnt
@@ -330,6 +335,8 @@ def test_biased_attention_prompt_portions_and_single_tokens(lib, dtype, H, G, D,
     for splits in ([n], [1] * n, [2, 2, 7, 1, 16, 3, 59], [70] + [1] * 20, [17, 2, 2, 69]):
         got, _ = _run_attn(lib, X, w, dtype, splits, H, G, D, E, scale, far, temp, eps)
         assert close(got, want, tol), splits
+    got, _ = _run_attn(lib, X, w, dtype, [40] + [1] * 50, H, G, D, E, scale, far, temp, eps, split_keys=False)
+    assert close(got, want, tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -250,7 +250,7 @@ class UmbSeqWork(C.Structure):
                 ("mix", C.c_void_p), ("act", C.c_void_p), ("y", C.c_void_p), ("logits", C.c_void_p),
                 ("Tmax", C.c_int32), ("Rmax", C.c_int32), ("moe_sel", C.c_void_p), ("moe_wt", C.c_void_p),
                 ("moe_pos", C.c_void_p), ("moe_tiles", C.c_void_p), ("moe_xs", C.c_void_p), ("moe_act", C.c_void_p),
-                ("moe_y", C.c_void_p), ("moe_max_tiles", C.c_int64)]
+                ("moe_y", C.c_void_p), ("moe_max_tiles", C.c_int64), ("aux_floats", C.c_int64)]
 
 
 class UmbSeqStep(C.Structure):
@@ -297,11 +297,11 @@ SEQ_SIGNATURES = {
     "umb_mingru_scratch_floats": [_I, _I, _I],
     "umb_mingru_scan": [_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _P, _L, _I],
     "umb_lin_scan": [_P, _P, _P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _F],
-    "umb_ssd_prep": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
+    "umb_ssd_prep": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I],
     "umb_ssd_conv_update": [_P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
     "umb_ssd_gate": [_P, _I, _P, _P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I],
     "umb_bsa_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I],
-    "umb_bsa_attend": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _I],
+    "umb_bsa_attend": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P, _L, _I],
     "umb_bsa_attend_tiled": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I],
     "umb_bsa_attend_tiled_ok": [_I, _I, _I, _I, _I],
     "umb_moe_route_softmax": [_P, _P, _P, _P, _I, _I, _I],

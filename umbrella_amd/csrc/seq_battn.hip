@@ -55,10 +55,12 @@ __global__ __launch_bounds__(NW * 64) void bsa_attend_kernel(typename El<P>::typ
                                                              const float* __restrict__ proj, int ld, int gate_col,
                                                              const float* __restrict__ bias, int n_dist,
                                                              const int* __restrict__ pos, const int* __restrict__ slot_, int H,
-                                                             int G, int D, int E, int window, float scale, float out_scale) {
+                                                             int G, int D, int E, int window, float scale, float out_scale,
+                                                             float* __restrict__ part, int nsplit) {
   typedef typename El<P>::type El_;
   extern __shared__ float lds[];
   constexpr int KB = 8;
+  const int split = blockIdx.z;                         // nsplit > 1: the workgroup takes every nsplit-th group of NW rounds
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int Dp = (D + 3) & ~3, Ep = (E + 3) & ~3, Mp = Dp > Ep ? Dp : Ep;
   // [RH][Dp] queries (later [NW][RH][Ep] partial sums), [NW][2 RH] maxima and denominators, per wave [RH][64] weights + offsets
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(NW * 64) void bsa_attend_kernel(typename El<P>::typ
   int dcl[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) dcl[c] = lane + 64 * c < E ? lane + 64 * c : E - 1;
-  for (int base = wave * 64; base < n_keys; base += NW * 64) {
+  for (int base = (split * NW + wave) * 64; base < n_keys; base += nsplit * NW * 64) {
     const int kx = base + lane;
     float s[RH];
 #pragma unroll
@@ -192,8 +194,45 @@ __global__ __launch_bounds__(NW * 64) void bsa_attend_kernel(typename El<P>::typ
       o += lds[(w * RH + r) * Ep + d] * f;
       L += ml_s[(w * RH + r) * 2 + 1] * f;
     }
+    if (nsplit > 1) {                                  // partial result of this split: [t][h][split][E + 2] = o.., M, L
+      float* pr = part + (((long)t * H + h0 + r) * nsplit + split) * (E + 2);
+      pr[d] = o;
+      if (d == 0) { pr[E] = M; pr[E + 1] = L; }
+      continue;
+    }
     const float gt = gate_col >= 0 ? 1.f / (1.f + expf(-proj[(long)t * ld + gate_col + h0 + r])) : 1.f;
     stf<P>(out + (long)t * ldo + (long)(h0 + r) * E + d, out_scale * gt * (o / L));
+  }
+}
+
+// the splits of one (token, head) merged: lane s holds split s's maximum and denominator (a split that had no key carries
+// M = -inf, L = 0), the factors go round by shuffles, every sum runs over the splits in order
+template <typename P>
+__global__ __launch_bounds__(64) void bsa_merge_kernel(typename El<P>::type* __restrict__ out, int ldo, const float* __restrict__ part,
+                                                       const float* __restrict__ proj, int ld, int gate_col, int H, int E,
+                                                       int nsplit, float out_scale) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* pr = part + ((long)t * H + h) * nsplit * (E + 2);
+  const float ms = lane < nsplit ? pr[lane * (E + 2) + E] : -INFINITY;
+  const float ls = lane < nsplit ? pr[lane * (E + 2) + E + 1] : 0.f;
+  const float gt = gate_col >= 0 ? 1.f / (1.f + expf(-proj[(long)t * ld + gate_col + h])) : 1.f;
+  const float M = wave_max(ms);
+  const float fs = ms == -INFINITY ? 0.f : expf(ms - M);
+  float L = 0.f, f[16];
+#pragma unroll
+  for (int s = 0; s < 16; ++s) {
+    f[s] = __shfl(fs, s, 64);
+    L += __shfl(ls * fs, s, 64);
+  }
+  const float c = out_scale * gt / L;
+  for (int d = lane; d < E; d += 64) {
+    float v[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) v[s] = pr[(s < nsplit ? s : nsplit - 1) * (E + 2) + d];
+    float o = 0.f;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) o += s < nsplit ? v[s] * f[s] : 0.f;
+    stf<P>(out + (long)t * ldo + (long)h * E + d, o * c);
   }
 }
 
@@ -215,7 +254,8 @@ extern "C" int umb_bsa_prep(float* q, const UmbPagedKV* kv, const float* proj, i
 
 extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
                               const float* bias, int n_dist, const int* pos, const int* slot, int T, int H, int G, int D, int E,
-                              int window, float scale, float out_scale, int dtype, hipStream_t st) {
+                              int window, float scale, float out_scale, float* scratch, long scratch_floats, int dtype,
+                              hipStream_t st) {
   if (T < 1 || H < 1 || G < 1 || H % G || D < 1 || E < 1 || E > 64 * BSA_MAXC || window < 1 || !out || !q || !bsa_kv_ok(kv) ||
       !pos || !slot || ldo < H * E || (bias && n_dist < 1) || (gate_col >= 0 && (!proj || ld < gate_col + H)))
     return UMB_EINVAL;
@@ -224,8 +264,17 @@ extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPaged
   // heads of one workgroup: query heads of one key/value head, as many as divide the group and fit the register budget
   int rh = nc <= 2 ? 8 : 4;
   while (rh > 1 && hpg % rh) rh >>= 1;
-  const dim3 grid(T, H / rh);
-  int nw = (long)T * (H / rh) < 1024 ? 16 : 4;
+  // A handful of (token, head block) items leaves most of the chip idle while each walks all its keys: with scratch for the
+  // partial results the keys of an item are dealt to several workgroups (whole groups of four 64-key rounds by number, so the
+  // order of every sum is a function of the position and of the step's row count only) and merged by a second launch.
+  const long items = (long)T * (H / rh);
+  int nsplit = 1;
+  if (scratch && items <= 64) {                          // fewer than ~2048 waves in all with sixteen waves per item
+    nsplit = (int)(512 / items) < 16 ? (int)(512 / items) : 16;
+    while (nsplit > 1 && (long)T * H * nsplit * (E + 2) > scratch_floats) nsplit >>= 1;
+  }
+  const dim3 grid(T, H / rh, nsplit);
+  int nw = (nsplit > 1 || items >= 1024) ? 4 : 16;
   auto lds_of = [&](int w) { return ((size_t)w * rh * Mp + (size_t)w * 2 * rh + (size_t)w * (rh * 64 + 128)) * sizeof(float); };
   if (nw == 16 && lds_of(16) > 128 * 1024) nw = 4;
   if (lds_of(nw) > 160 * 1024) return UMB_EINVAL;
@@ -234,7 +283,7 @@ extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPaged
   do {                                                                                                                      \
     if (ensure_dynamic_lds<bsa_attend_kernel<P, RH, NC, NW>>(lds) != UMB_OK) return UMB_EHIP;                               \
     hipLaunchKernelGGL((bsa_attend_kernel<P, RH, NC, NW>), grid, dim3(NW * 64), lds, st, (El_*)out, ldo, q, *kv, proj, ld,  \
-                       gate_col, bias, n_dist, pos, slot, H, G, D, E, window, scale, out_scale);                            \
+                       gate_col, bias, n_dist, pos, slot, H, G, D, E, window, scale, out_scale, scratch, nsplit);           \
   } while (0)
 #define BSA_NW(RH, NC)                                                                                                      \
   if (nw == 16) BSA_LAUNCH(RH, NC, 16); else BSA_LAUNCH(RH, NC, 4)
@@ -245,6 +294,9 @@ extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPaged
     if (nc <= 1) { BSA_RH(1) }
     else if (nc <= 2) { BSA_RH(2) }
     else { if (rh == 4) { BSA_NW(4, 4); } else if (rh == 2) { BSA_NW(2, 4); } else { BSA_NW(1, 4); } }
+    if (nsplit > 1)
+      hipLaunchKernelGGL(bsa_merge_kernel<P>, dim3(T, H), dim3(64), 0, st, (El_*)out, ldo, scratch, proj, ld, gate_col, H, E, nsplit,
+                         out_scale);
   })
 #undef BSA_RH
 #undef BSA_NW

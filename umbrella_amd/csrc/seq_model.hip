@@ -127,13 +127,20 @@ static int mix_attn_ssd(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
   if (s->max_len >= 16 && umb_bsa_attend_tiled_ok(H, G, D, E, dt))
     SEQ_TRY(umb_bsa_attend_tiled(ws->mix, ldo, q, &ly.kv, ws->proj, ld, gate_col, ly.dist_bias, ly.n_dist, s->seq_slot, s->seq_row0,
                                  s->seq_pos0, s->seq_len, s->B, s->max_len, H, G, D, E, ly.window, ly.scale, ly.mix_scale_a, dt, st));
-  else
+  else {
+    // what the step leaves free of aux holds the partial results of split keys (the state-space part below uses sx / alpha
+    // after the attention is done, so its region may be used too, but the queries may not)
+    float* spare = q + (size_t)T * H * D;
+    const long spare_floats = ws->aux_floats - (long)T * H * D;
     SEQ_TRY(umb_bsa_attend(ws->mix, ldo, q, &ly.kv, ws->proj, ld, gate_col, ly.dist_bias, ly.n_dist, s->pos, s->slot, T, H, G, D, E,
-                           ly.window, ly.scale, ly.mix_scale_a, dt, st));
+                           ly.window, ly.scale, ly.mix_scale_a, spare_floats > 0 ? spare : nullptr, spare_floats, dt, st));
+  }
+  const int single = s->max_len == 1;                       // one token per sequence: the ring is updated inside prep
   SEQ_TRY(umb_ssd_prep(sx, lds, alpha, ws->proj, ld, col0, ly.s_conv, ly.s_conv_b, ly.s_conv_state, ly.s_dt_bias, ly.s_a_log, s->pos,
-                       s->slot, T, sH, sDv, sG, N, ly.s_taps, dt, st));
-  SEQ_TRY(umb_ssd_conv_update(ly.s_conv_state, ws->proj, ld, col0 + inner, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B,
-                              C, ly.s_taps, st));
+                       s->slot, T, sH, sDv, sG, N, ly.s_taps, single, dt, st));
+  if (!single)
+    SEQ_TRY(umb_ssd_conv_update(ly.s_conv_state, ws->proj, ld, col0 + inner, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len,
+                                s->B, C, ly.s_taps, st));
   SEQ_TRY(umb_lin_scan(ws->o, ly.state, sx + inner + sG * N, lds, sx + inner, lds, sx, lds, alpha, 1, sG, s->seq_slot, s->seq_row0,
                        s->seq_pos0, s->seq_len, s->B, sH, N, sDv, 1.f, st));
   void* right = static_cast<char*>(ws->mix) + (size_t)H * E * seq_elem_bytes(dt);

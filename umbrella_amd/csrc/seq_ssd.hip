@@ -4,7 +4,8 @@
 // bias) per head, and B / C are shared by the heads of a group.  The recurrence is the linear scan of seq_gla.hip with
 // k = B, v = dt x, q = C and one decay per head; this file holds what surrounds it:
 //   prep         convolution (inputs of earlier steps from the sequence's state ring) + bias + silu, dt, decay, dt x
-//   conv_update  the step's last taps - 1 raw inputs into the state ring (after prep has read it)
+//   conv_update  the step's last taps - 1 raw inputs into the state ring (after prep has read it); steps of one token per
+//                sequence do this inside prep
 //   gate         y = o + D x, times silu(z), unit RMS in equal parts of the row, times a weight and a constant, rounded
 // Everything is fp32 (the convolution too); the only rounding is the gated, normed output that feeds the output projection.
 // The convolution sums its taps oldest first whatever their source, so a position's value does not depend on where a prompt
@@ -18,9 +19,10 @@ __global__ __launch_bounds__(256) void ssd_prep_kernel(float* __restrict__ sx, i
                                                        const float* __restrict__ proj, int ld, int col0,
                                                        const typename El<P>::type* __restrict__ conv_w,
                                                        const typename El<P>::type* __restrict__ conv_b,
-                                                       const float* __restrict__ conv_state, const float* __restrict__ dt_bias,
+                                                       float* __restrict__ conv_state, const float* __restrict__ dt_bias,
                                                        const float* __restrict__ a_log, const int* __restrict__ pos,
-                                                       const int* __restrict__ slot_, int H, int Dv, int G, int N, int taps) {
+                                                       const int* __restrict__ slot_, int H, int Dv, int G, int N, int taps,
+                                                       int update) {
   const int t = blockIdx.x, idx = blockIdx.y * 256 + threadIdx.x;
   const int inner = H * Dv, C = inner + 2 * G * N;
   const float* pr = proj + (long)t * ld + col0;
@@ -41,6 +43,9 @@ __global__ __launch_bounds__(256) void ssd_prep_kernel(float* __restrict__ sx, i
     }
     acc += ldf<P>(conv_w + (long)idx * taps + j) * in;
   }
+  // steps of one token per sequence: this thread is the only one that touches the ring of (slot, channel); the row of the
+  // token's position held the oldest tap, which has been read above
+  if (update && taps > 1) conv_state[((long)slot * (taps - 1) + p % (taps - 1)) * C + idx] = proj[(long)t * ld + col0 + inner + idx];
   const float v = siluf_(acc);
   if (idx < inner) {
     const int h = idx / Dv;
@@ -88,8 +93,9 @@ __global__ __launch_bounds__(256) void ssd_gate_kernel(typename El<P>::type* __r
 }
 
 extern "C" int umb_ssd_prep(float* sx, int lds, float* alpha, const float* proj, int ld, int col0, const void* conv_w,
-                            const void* conv_b, const float* conv_state, const float* dt_bias, const float* a_log, const int* pos,
-                            const int* slot, int T, int H, int Dv, int G, int N, int taps, int dtype, hipStream_t st) {
+                            const void* conv_b, float* conv_state, const float* dt_bias, const float* a_log, const int* pos,
+                            const int* slot, int T, int H, int Dv, int G, int N, int taps, int update_state, int dtype,
+                            hipStream_t st) {
   if (T < 1 || H < 1 || Dv < 1 || G < 1 || N < 1 || H % G || taps < 1 || !sx || !alpha || !proj || !conv_w || !dt_bias ||
       !a_log || !pos || !slot || (taps > 1 && !conv_state))
     return UMB_EINVAL;
@@ -98,7 +104,7 @@ extern "C" int umb_ssd_prep(float* sx, int lds, float* alpha, const float* proj,
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
     hipLaunchKernelGGL(ssd_prep_kernel<P>, dim3(T, (C + H + 255) / 256), dim3(256), 0, st, sx, lds, alpha, proj, ld, col0,
-                       (const E*)conv_w, (const E*)conv_b, conv_state, dt_bias, a_log, pos, slot, H, Dv, G, N, taps);
+                       (const E*)conv_w, (const E*)conv_b, conv_state, dt_bias, a_log, pos, slot, H, Dv, G, N, taps, update_state);
   })
   UMB_LAUNCH_CHECK();
   return UMB_OK;

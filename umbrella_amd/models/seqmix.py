@@ -282,7 +282,7 @@ class SeqMixLM(LLMBase):
             for k in ("moe_sel", "moe_wt", "moe_pos", "moe_tiles", "moe_xs", "moe_act", "moe_y"):
                 setattr(ws, k, b[k].data_ptr())
             ws.moe_max_tiles = tiles
-        ws.Tmax, ws.Rmax = T, R
+        ws.Tmax, ws.Rmax, ws.aux_floats = T, R, b["aux"].numel()
         self.ws_tokens, self.logit_rows = T, R
 
     @property
