@@ -221,16 +221,26 @@ int umb_lin_scan(float* o, float* state, const float* q, int ldq, const float* k
  * [z (H Dv) | x (H Dv) | B (G N) | C (G N) | dt (H)].  prep: x, B, C through a causal convolution per channel (w [C][taps],
  * last column the token's own, bias b, inputs of earlier steps from conv_state fp32 [slots][taps - 1][C], the input of
  * position p in row p % (taps - 1)) and silu; dt = softplus(dt + dt_bias[h]); sx fp32 [T][lds] = [dt x | B | C | x],
- * alpha [T][H] = exp(-exp(a_log[h]) dt).  conv_update, launched after prep, stores the step's last raw inputs; with
+ * alpha [T][H] = exp(-exp(a_log[h]) dt), log_alpha [T][H] (may be null) its logarithm.  conv_update, launched after prep, stores the step's last raw inputs; with
  * update_state (steps of ONE token per sequence only) prep stores the token's input itself and conv_update is not needed.
  * The recurrence itself is umb_lin_scan (k = B, v = dt x, q = C).
  * gate: y = o + d_skip[h] x, times silu(z), unit RMS in `norm_groups` equal parts of the H Dv row, times w, times
  * out_scale, in `dtype` at out[t ldo + ...]. */
-int umb_ssd_prep(float* sx, int lds, float* alpha, const float* proj, int ld, int col0, const void* conv_w, const void* conv_b,
+int umb_ssd_prep(float* sx, int lds, float* alpha, float* log_alpha, const float* proj, int ld, int col0, const void* conv_w,
+                 const void* conv_b,
                  float* conv_state, const float* dt_bias, const float* a_log, const int* pos, const int* slot, int T, int H,
                  int Dv, int G, int N, int taps, int update_state, int dtype, umb_stream_t stream);
 int umb_ssd_conv_update(float* conv_state, const float* proj, int ld, int col0, const int* seq_slot, const int* seq_row0,
                         const int* seq_pos0, const int* seq_len, int B, int C, int taps, umb_stream_t stream);
+/* The recurrence of umb_lin_scan with one decay per head (given as its logarithm), for stretches of many tokens: chunks of 64
+ * tokens run side by side -- chunk summaries, a pass over the chunks that leaves every chunk's start state and the final state
+ * in the slot, then all read-outs (qscale 1).  scratch fp32 of at least umb_ssd_scan_chunked_floats(..) floats (0: the shape is
+ * not covered; no stream argument).  Equal to the token-by-token scan to fp32 rounding. */
+long umb_ssd_scan_chunked_floats(int B, int max_len, int H, int N, int P);
+int umb_ssd_scan_chunked(float* o, float* state, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                         const float* log_alpha, int qk_heads, const int* seq_slot, const int* seq_row0, const int* seq_pos0,
+                         const int* seq_len, int B, int max_len, int H, int N, int P, float* scratch, long scratch_floats,
+                         umb_stream_t stream);
 int umb_ssd_gate(void* out, int ldo, const float* o, const float* sx, int lds, int x_col, const float* proj, int ld, int z_col,
                  const float* d_skip, const void* w, int T, int H, int Dv, int norm_groups, float eps, float out_scale, int dtype,
                  umb_stream_t stream);

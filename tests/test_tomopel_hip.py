@@ -172,7 +172,7 @@ def _ssd_weights(width, H, Dv, N, G, taps, seed):
                 d_skip=1.0 + rnd((H,), seed + 5, 0.2), norm_w=1.0 + rnd((inner,), seed + 6, 0.1))
 
 
-def _run_ssd(lib, X, w, dtype, splits, H, Dv, N, G, NG, taps, eps, scale=1.0, slot=1, state=None, conv=None, col0=3):
+def _run_ssd(lib, X, w, dtype, splits, H, Dv, N, G, NG, taps, eps, scale=1.0, slot=1, state=None, conv=None, col0=3, chunked=True):
     """prep + state ring + scan + gate through their entry points, the sequence cut into `splits`; returns the gated, normed
     rows [n, H Dv] (what the output projection reads)"""
     from umbrella_amd import _lib
@@ -189,16 +189,23 @@ def _run_ssd(lib, X, w, dtype, splits, H, Dv, N, G, NG, taps, eps, scale=1.0, sl
         proj = dev(proj_all[at:at + cnt])
         sx = torch.zeros(cnt, lds + 1, dtype=torch.float32, device="cuda:0")
         alpha = torch.zeros(cnt, H, dtype=torch.float32, device="cuda:0")
+        la = torch.zeros(cnt, H, dtype=torch.float32, device="cuda:0")
         o = torch.zeros(cnt, inner, dtype=torch.float32, device="cuda:0")
         out = torch.zeros(cnt, inner + 2, dtype=dtype, device="cuda:0")
         single = int(cnt == 1)                                          # as the forward does: one launch for single tokens
-        _lib.seq_call("umb_ssd_prep", sx, lds + 1, alpha, proj, ld, col0, dev(w["conv_w"], dtype), dev(w["conv_b"], dtype), conv,
+        _lib.seq_call("umb_ssd_prep", sx, lds + 1, alpha, la, proj, ld, col0, dev(w["conv_w"], dtype), dev(w["conv_b"], dtype), conv,
                       f32("dt_bias"), f32("a_log"), st.d["pos"], st.d["slot"], cnt, H, Dv, G, N, taps, single, code(dtype))
         if not single:
             _lib.seq_call("umb_ssd_conv_update", conv, proj, ld, col0 + inner, st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"],
                           st.d["seq_len"], 1, C, taps)
-        _lib.seq_call("umb_lin_scan", o, state, sx[:, inner + gn:], lds + 1, sx[:, inner:], lds + 1, sx, lds + 1, alpha, 1, G,
-                      st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, H, N, Dv, 1.0)
+        need = lib.umb_ssd_scan_chunked_floats(1, cnt, H, N, Dv) if cnt >= 64 and chunked else 0
+        if need > 0:                                                    # as the forward does: long stretches in chunks
+            scratch = torch.zeros(need, dtype=torch.float32, device="cuda:0")
+            _lib.seq_call("umb_ssd_scan_chunked", o, state, sx[:, inner + gn:], lds + 1, sx[:, inner:], lds + 1, sx, lds + 1, la, G,
+                          st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, cnt, H, N, Dv, scratch, need)
+        else:
+            _lib.seq_call("umb_lin_scan", o, state, sx[:, inner + gn:], lds + 1, sx[:, inner:], lds + 1, sx, lds + 1, alpha, 1, G,
+                          st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, H, N, Dv, 1.0)
         _lib.seq_call("umb_ssd_gate", out, inner + 2, o, sx, lds + 1, C, proj, ld, col0, f32("d_skip"), dev(w["norm_w"], dtype), cnt, H,
                       Dv, NG, eps, scale, code(dtype))
         outs.append(out[:, :inner].clone())
@@ -227,6 +234,24 @@ def test_state_space_prompt_portions_and_single_tokens(lib, dtype, H, Dv, N, G, 
         got = _run_ssd(lib, X, w, dtype, splits, H, Dv, N, G, NG, taps, eps)
         assert close(got, want, tol), splits
     assert close(_run_ssd(lib, X, w, dtype, [n], H, Dv, N, G, NG, taps, eps, scale=0.25), 0.25 * want, tol)
+
+
+@pytest.mark.parametrize("H,Dv,N,G,NG,taps", [(3, 4, 5, 1, 1, 3), (4, 32, 64, 2, 4, 4), (2, 20, 130, 1, 2, 3), (2, 70, 16, 2, 1, 2),
+                                              (1, 136, 24, 1, 1, 4)])
+def test_state_space_long_stretches_in_chunks(lib, H, Dv, N, G, NG, taps):
+    """stretches of 64 tokens and more take the chunked form (whole and partial chunks, a carried state in front, single tokens
+    behind); against the oracle and against the token-by-token scan"""
+    n, width, eps = 210, 24, 1e-5
+    w = _ssd_weights(width, H, Dv, N, G, taps, seed=H + N)
+    w["dt_bias"] = w["dt_bias"] - 1.5                                   # slow decays: the state remembers across chunks
+    X = rnd((n, width), 5)
+    want = _ssd_oracle(X, w, torch.float32, H, Dv, N, G, NG, eps)
+    serial = _run_ssd(lib, X, w, torch.float32, [n], H, Dv, N, G, NG, taps, eps, chunked=False)
+    assert close(serial, want, F32_TOL)
+    for splits in ([n], [64, 146], [3, 128, 65, 1, 1, 12], [100, 1, 109], [65] + [1] * 81 + [64]):
+        got = _run_ssd(lib, X, w, torch.float32, splits, H, Dv, N, G, NG, taps, eps)
+        assert close(got, want, F32_TOL) and close(got, serial, F32_TOL), splits
+    assert close(_run_ssd(lib, X, w, torch.bfloat16, [n], H, Dv, N, G, NG, taps, eps), _ssd_oracle(X, w, torch.bfloat16, H, Dv, N, G, NG, eps), 2e-2)
 
 
 def test_state_space_slot_is_reused_without_leaking(lib):
@@ -574,6 +599,28 @@ def test_model_long_decoding_and_first_tokens(lib):
     got = torch.cat(rows)
     assert rel_err(got, want) < F32_TOL
     assert rel_err(got[:3], want[:3]) < F32_TOL
+
+
+@pytest.mark.parametrize("name", ["mixed", "single"])
+def test_model_long_prompt_in_one_step_and_in_portions(lib, name):
+    """fp32: a 200-token prompt (state-space chunks of 64, minGRU pieces from 128 tokens on, matrix-free attention) whole, in two
+    long portions, and with a second sequence of another length beside it, against the oracle"""
+    from tomopel_helpers import BIAS_ROWS, CONFIGS, build
+    cfgd = CONFIGS[name]
+    m, sd = build(cfgd, torch.float32, seed=13, page=4, batch=3, max_tokens=1200, max_length=512, bias_rows=BIAS_ROWS[name])
+    toks, other = tokens(200, cfgd["vocab"], 21), tokens(77, cfgd["vocab"], 22)
+    want, want2 = _oracle_logits(cfgd, sd, toks), _oracle_logits(cfgd, sd, other)
+    rows = list(range(0, 200, 7)) + [199]
+    m.open("a")
+    assert rel_err(m.forward_batch([("a", toks)], want=[rows]), want[rows]) < F32_TOL
+    m.open("b")
+    first = m.forward_batch([("b", toks[:130])], want=[[r for r in rows if r < 130]]).clone()
+    second = m.forward_batch([("b", toks[130:])], want=[[r - 130 for r in rows if r >= 130]]).clone()
+    assert rel_err(torch.cat([first, second]), want[rows]) < F32_TOL
+    m.close("a"), m.close("b")
+    m.open("c"), m.open("d")
+    both = m.forward_batch([("c", other), ("d", toks)], want=[[76], rows])
+    assert rel_err(both[:1], want2[76:77]) < F32_TOL and rel_err(both[1:], want[rows]) < F32_TOL
 
 
 def test_model_decode_steps_replayed_as_graphs_equal_eager_launches(lib):

@@ -297,7 +297,9 @@ SEQ_SIGNATURES = {
     "umb_mingru_scratch_floats": [_I, _I, _I],
     "umb_mingru_scan": [_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _P, _L, _I],
     "umb_lin_scan": [_P, _P, _P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _F],
-    "umb_ssd_prep": [_P, _I, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I],
+    "umb_ssd_prep": [_P, _I, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I],
+    "umb_ssd_scan_chunked_floats": [_I, _I, _I, _I, _I],
+    "umb_ssd_scan_chunked": [_P, _P, _P, _I, _P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _L],
     "umb_ssd_conv_update": [_P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
     "umb_ssd_gate": [_P, _I, _P, _P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I],
     "umb_bsa_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I],
@@ -311,7 +313,8 @@ SEQ_SIGNATURES = {
     "umb_sample_rows": [_P, _P, _I, _I, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P],
     "umb_seq_version": [],
 }
-_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok", "umb_seq_resid_canon_step_ok", "umb_bsa_attend_tiled_ok", "umb_mingru_scratch_floats"}          # predicates: no stream argument, the value is the answer
+_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok", "umb_seq_resid_canon_step_ok", "umb_bsa_attend_tiled_ok", "umb_mingru_scratch_floats",
+                  "umb_ssd_scan_chunked_floats"}          # predicates: no stream argument, the value is the answer
 _seq_lib = None
 
 

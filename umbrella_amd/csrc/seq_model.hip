@@ -119,9 +119,12 @@ static int mix_attn_ssd(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
   const int gate_col = H * D + G * D + G * E, col0 = gate_col + H;
   const int inner = sH * sDv, C = inner + 2 * sG * N, lds = C + inner, ldo = H * E + inner;
   if (ld != col0 + 2 * inner + 2 * sG * N + sH || ly.out.K != ldo || !ly.state) return UMB_EINVAL;
-  float* q = ws->aux;                                        // [T][H D] | [T][lds] | [T][sH]
+  float* q = ws->aux;                                        // [T][H D] | [T][lds] | [T][sH] | [T][sH] | scratch
   float* sx = q + (size_t)T * H * D;
   float* alpha = sx + (size_t)T * lds;
+  float* log_alpha = alpha + (size_t)T * sH;
+  float* spare2 = log_alpha + (size_t)T * sH;
+  const long spare2_floats = ws->aux_floats - (long)(spare2 - ws->aux);
   SEQ_TRY(umb_bsa_prep(q, &ly.kv, ws->proj, ld, ly.q_norm, ly.k_norm, s->pos, s->slot, T, H, G, D, E, ly.temp_coef, ly.temp_every,
                        m->eps, dt, st));
   if (s->max_len >= 16 && umb_bsa_attend_tiled_ok(H, G, D, E, dt))
@@ -136,13 +139,19 @@ static int mix_attn_ssd(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
                            ly.window, ly.scale, ly.mix_scale_a, spare_floats > 0 ? spare : nullptr, spare_floats, dt, st));
   }
   const int single = s->max_len == 1;                       // one token per sequence: the ring is updated inside prep
-  SEQ_TRY(umb_ssd_prep(sx, lds, alpha, ws->proj, ld, col0, ly.s_conv, ly.s_conv_b, ly.s_conv_state, ly.s_dt_bias, ly.s_a_log, s->pos,
+  SEQ_TRY(umb_ssd_prep(sx, lds, alpha, log_alpha, ws->proj, ld, col0, ly.s_conv, ly.s_conv_b, ly.s_conv_state, ly.s_dt_bias, ly.s_a_log, s->pos,
                        s->slot, T, sH, sDv, sG, N, ly.s_taps, single, dt, st));
   if (!single)
     SEQ_TRY(umb_ssd_conv_update(ly.s_conv_state, ws->proj, ld, col0 + inner, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len,
                                 s->B, C, ly.s_taps, st));
-  SEQ_TRY(umb_lin_scan(ws->o, ly.state, sx + inner + sG * N, lds, sx + inner, lds, sx, lds, alpha, 1, sG, s->seq_slot, s->seq_row0,
-                       s->seq_pos0, s->seq_len, s->B, sH, N, sDv, 1.f, st));
+  // stretches of many tokens: the recurrence in chunks side by side, where the shape is covered and the scratch suffices
+  const long need = s->max_len >= 64 ? umb_ssd_scan_chunked_floats(s->B, s->max_len, sH, N, sDv) : 0;
+  if (need > 0 && need <= spare2_floats && (long)s->B * sH <= 65535)
+    SEQ_TRY(umb_ssd_scan_chunked(ws->o, ly.state, sx + inner + sG * N, lds, sx + inner, lds, sx, lds, log_alpha, sG, s->seq_slot,
+                                 s->seq_row0, s->seq_pos0, s->seq_len, s->B, s->max_len, sH, N, sDv, spare2, spare2_floats, st));
+  else
+    SEQ_TRY(umb_lin_scan(ws->o, ly.state, sx + inner + sG * N, lds, sx + inner, lds, sx, lds, alpha, 1, sG, s->seq_slot, s->seq_row0,
+                         s->seq_pos0, s->seq_len, s->B, sH, N, sDv, 1.f, st));
   void* right = static_cast<char*>(ws->mix) + (size_t)H * E * seq_elem_bytes(dt);
   return umb_ssd_gate(right, ldo, ws->o, sx, lds, C, ws->proj, ld, col0, ly.s_d, ly.s_norm, T, sH, sDv, ly.s_norm_groups, m->eps,
                       ly.mix_scale_b, dt, st);

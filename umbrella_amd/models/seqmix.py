@@ -252,9 +252,13 @@ class SeqMixLM(LLMBase):
             elif m.kind == "mingru":
                 ask(mix=m.dim, aux=3 * m.dim + m.dim // 16 + 1)     # aux: piece summaries and start states of long stretches
             elif m.kind == "attention_ssd":
-                # aux: queries | convolved [dt x | B | C | x] | decays; o: the scan's read-out; mix: [attention | state space]
+                # aux: queries | convolved [dt x | B | C | x] | decays and their logarithms | chunk states of the chunked scan
+                # (one [state, vdim] matrix per head and 64 tokens, and room for a few partial chunks); o: the scan's
+                # read-out; mix: [attention | state space]
                 inner = m.s_heads * m.s_vdim
-                ask(aux=m.heads * m.dim + 2 * inner + 2 * m.s_groups * m.s_state + m.s_heads, o=inner, mix=m.heads * m.vdim + inner)
+                chunk = m.s_heads * (m.s_state * m.s_vdim + 1)
+                ask(aux=m.heads * m.dim + 2 * inner + 2 * m.s_groups * m.s_state + 2 * m.s_heads + (chunk + 63) // 64 + (8 * chunk) // T + 1,
+                    o=inner, mix=m.heads * m.vdim + inner)
             else:
                 ask(aux=m.heads * m.dim, o=m.heads * m.vdim, mix=m.heads * m.vdim)
             if ly.ff_kind == "moe":
