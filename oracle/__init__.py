@@ -4,7 +4,7 @@ TEST INFRASTRUCTURE ONLY.  This package is a plain torch-CPU / numpy
 restatement of the reference algorithm (Infini-AI-Lab/UMbreLLa @ 2025-02-16)
 for the draft-expand / verify path.  Only ``tests/``, ``__graft_entry__.smoke()``
 and ``bench.py``'s ``cpu_baseline`` leg may import it -- and there only as the
-checker, never as the thing measured or shipped.  The product
+yardstick, never as the thing measured or shipped.  The product
 (``umbrella_amd``) never imports ``oracle`` and raises when its HIP library is
 missing.
 

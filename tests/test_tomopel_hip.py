@@ -348,6 +348,7 @@ def _attn_oracle(X, w, dtype, H, G, D, E, scale, far, temp, eps):
 @pytest.mark.parametrize("H,G,D,E,rows,far,temp", [(4, 2, 8, 6, 12, 40, (0.3, 8)), (3, 1, 7, 9, 4, 9, (0.0, 0)), (2, 2, 16, 16, 7, 25, (0.5, 1)),
                                                    (8, 2, 32, 64, 32, 70, (0.2, 16)), (6, 3, 24, 130, 9, 1000, (0.1, 5)),
                                                    (12, 1, 40, 48, 10, 33, (0.2, 7)), (4, 4, 136, 144, 6, 20, (0.0, 0)),
+                                                   (2, 1, 16, 400, 8, 30, (0.1, 9)),
                                                    (1, 1, 8, 200, 16, 16, (1.0, 64))])
 def test_biased_attention_prompt_portions_and_single_tokens(lib, dtype, H, G, D, E, rows, far, temp):
     """every bucket of the table is reached (far < n for most shapes), the temperature steps several times, keys sit on both

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void bsa_prep_kernel(float* __restrict__ q, Um
   }
 }
 
-constexpr int BSA_MAXC = 4;      // value columns per lane: E <= 256
+constexpr int BSA_MAXC = 8;      // value columns per lane: E <= 512
 
 template <typename P, int RH, int NC, int NW>
 __global__ __launch_bounds__(NW * 64) void bsa_attend_kernel(typename El<P>::type* __restrict__ out, int ldo,
@@ -262,7 +262,7 @@ extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPaged
   const int hpg = H / G, nc = (E + 63) / 64;
   const int Dp = (D + 3) & ~3, Ep = (E + 3) & ~3, Mp = Dp > Ep ? Dp : Ep;
   // heads of one workgroup: query heads of one key/value head, as many as divide the group and fit the register budget
-  int rh = nc <= 2 ? 8 : 4;
+  int rh = nc <= 2 ? 8 : (nc <= 4 ? 4 : 2);
   while (rh > 1 && hpg % rh) rh >>= 1;
   // A handful of (token, head block) items leaves most of the chip idle while each walks all its keys: with scratch for the
   // partial results the keys of an item are dealt to several workgroups (whole groups of four 64-key rounds by number, so the
@@ -293,7 +293,8 @@ extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPaged
     typedef typename El<P>::type El_;
     if (nc <= 1) { BSA_RH(1) }
     else if (nc <= 2) { BSA_RH(2) }
-    else { if (rh == 4) { BSA_NW(4, 4); } else if (rh == 2) { BSA_NW(2, 4); } else { BSA_NW(1, 4); } }
+    else if (nc <= 4) { if (rh == 4) { BSA_NW(4, 4); } else if (rh == 2) { BSA_NW(2, 4); } else { BSA_NW(1, 4); } }
+    else { if (rh == 2) { BSA_NW(2, 8); } else { BSA_NW(1, 8); } }
     if (nsplit > 1)
       hipLaunchKernelGGL(bsa_merge_kernel<P>, dim3(T, H), dim3(64), 0, st, (El_*)out, ldo, scratch, proj, ld, gate_col, H, E, nsplit,
                          out_scale);
