@@ -28,14 +28,21 @@ extern "C" {
 typedef struct ihipStream_t* umb_stream_t;   /* == hipStream_t */
 
 enum { UMB_SEQ_F16 = 0, UMB_SEQ_BF16 = 1, UMB_SEQ_F32 = 2 };
-enum { UMB_MIX_POOLED_WINDOW = 0, UMB_MIX_GLA = 1, UMB_MIX_LATENT = 2, UMB_MIX_MINGRU = 3, UMB_MIX_ATTN_SSD = 4 };
+enum { UMB_MIX_POOLED_WINDOW = 0, UMB_MIX_GLA = 1, UMB_MIX_LATENT = 2, UMB_MIX_MINGRU = 3, UMB_MIX_ATTN_SSD = 4,
+       UMB_MIX_RETENTION = 5, UMB_MIX_ATTN_MLSTM = 6 };
 /* feed-forward kinds: gated SiLU (W_down (silu(W_gate h) * W_up h)), PolyNorm (W_down polynorm(W_up h)), routed experts */
 enum { UMB_FF_GATED = 0, UMB_FF_POLYNORM = 1, UMB_FF_MOE = 2 };
-/* activation of a feed-forward / expert: silu(W_gate h) * (W_up h) over stacked [gate; up], or relu(W_up h)^2 (no gate) */
-enum { UMB_ACT_SILU_GATED = 0, UMB_ACT_RELU2 = 1 };
+/* activation of a feed-forward / expert: silu(W_gate h) * (W_up h) over stacked [gate; up], relu(W_up h)^2 (no gate), or the
+ * capped form g sigmoid(alpha g) (u + 1) with g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit) over stacked [gate; up] */
+enum { UMB_ACT_SILU_GATED = 0, UMB_ACT_RELU2 = 1, UMB_ACT_CLAMP_GLU = 2 };
 /* routing of experts: sigmoid scores that multiply the expert's input; or softmax scores, chosen with a correction added,
  * renormalised over the chosen ones, that multiply the expert's output */
-enum { UMB_ROUTE_SIGMOID_IN = 0, UMB_ROUTE_SOFTMAX_OUT = 1 };
+enum { UMB_ROUTE_SIGMOID_IN = 0, UMB_ROUTE_SOFTMAX_OUT = 1, UMB_ROUTE_TOP_LOGITS = 2 };
+/* UMB_ROUTE_TOP_LOGITS: the largest logits are chosen, the weights are the softmax over the chosen logits alone and multiply
+ * the experts' outputs */
+/* how a layer's sublayers meet the residual: one after the other (x + f(..) then x + g(..), the forms below), or BOTH reading the
+ * same x: x <- x + (mixer(norm1(x)) + ff(norm2(x))) */
+enum { UMB_BLOCK_SEQUENTIAL = 0, UMB_BLOCK_PARALLEL = 1 };
 
 /* W [N][K] row-major (as stored: out x in), optional bias [N]; applied as W x + b */
 typedef struct UmbSeqLinear { const void* w; const void* bias; int32_t N, K; } UmbSeqLinear;
@@ -251,21 +258,23 @@ int umb_ssd_gate(void* out, int ldo, const float* o, const float* sx, int lds, i
  * the heads; null: 1); cache K <- unit_rms(k) * w_k; cache V <- unit_rms(v) (no weight).
  * attend: score(i, j, h) = q_i . k_j * scale + bias[h][min(i - j, n_dist - 1)] over j <= i with i - j < window (bias fp32
  * [H][n_dist], null: none); softmax; out[t ldo + h E ..] = out_scale * sigmoid(gate[t][h]) * sum_j p_j v_j in `dtype`
- * (gate_col < 0: no gate).  scratch (fp32, may be null): with it, steps of few rows deal each row's keys to several workgroups
+ * (gate_col < 0: no gate).  softcap > 0: the scaled product is capped, softcap tanh(q . k scale / softcap), before the bias
+ * joins it.  scratch (fp32, may be null): with it, steps of few rows deal each row's keys to several workgroups
  * (as many as T H 16 (E + 2) floats allow, at most 16) and merge the partial results in a second launch. */
 int umb_bsa_prep(float* q, const UmbPagedKV* kv, const float* proj, int ld, const void* w_q, const void* w_k, const int* pos,
                  const int* slot, int T, int H, int G, int D, int E, float temp_coef, int temp_every, float eps, int dtype,
                  umb_stream_t stream);
 int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
                    const float* bias, int n_dist, const int* pos, const int* slot, int T, int H, int G, int D, int E, int window,
-                   float scale, float out_scale, float* scratch, long scratch_floats, int dtype, umb_stream_t stream);
+                   float scale, float out_scale, float softcap, float* scratch, long scratch_floats, int dtype,
+                   umb_stream_t stream);
 /* the same for steps that bring stretches of a sequence, on the matrix pipe (16-bit storage; umb_bsa_attend_tiled_ok says
  * 1 / 0 whether the kernel covers a shape and dtype; it has no stream): workgroups own 16 consecutive positions */
 int umb_bsa_attend_tiled_ok(int H, int G, int D, int E, int dtype);
 int umb_bsa_attend_tiled(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
                          const float* bias, int n_dist, const int* seq_slot, const int* seq_row0, const int* seq_pos0,
                          const int* seq_len, int B, int max_len, int H, int G, int D, int E, int window, float scale,
-                         float out_scale, int dtype, umb_stream_t stream);
+                         float out_scale, float softcap, int dtype, umb_stream_t stream);
 
 /* ---- routed experts, softmax form: scores = softmax(logits) over all experts; the `top` largest of score + correction
  * (correction fp32 [E], null: none; ties: the lower index) are chosen; wt = the chosen scores over (their sum + 1e-20). */
@@ -274,6 +283,70 @@ int umb_moe_route_softmax(int* sel, float* wt, const float* logits, const float*
 /* y[t] = (add ? y[t] : 0) + sum_k wt[t top + k] * ye[pos_of[t top + k]]  (k ascending) */
 int umb_moe_combine_weighted(float* y, const float* ye, const float* wt, const int* pos_of, int T, int W, int top, int add,
                              umb_stream_t stream);
+
+/* ---- the capped gated epilogue over stacked [gate; up] (N = 2 N'): out[T][N'] in `dtype` = g sigmoid(alpha g) (u + 1) with
+ * g = min(gate, limit), u = clamp(up, -limit, limit); dense and grouped forms of umb_seq_linear / umb_seq_linear_grouped */
+int umb_seq_linear_glu(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, float limit, float alpha,
+                       int dtype, umb_stream_t stream);
+int umb_seq_linear_grouped_glu(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows, long gs,
+                               int N, int K, float limit, float alpha, int dtype, umb_stream_t stream);
+
+/* ---- layers whose two sublayers read the same residual.  One launch between two layers:
+ *   embed_mode 0: x += y1 + y2;  1: x = embed[token] * embed_scale;  2: x += (y1 + y2) + embed[token] * embed_scale
+ * (y1 / y2 fp32 [T][W], either may be null), then h1 = x / rms(x) * (offset + w1) and h2 likewise with w2, in `dtype` (w1 / w2
+ * null: that output is not written). */
+int umb_blk_seam(float* x, void* h1, void* h2, const float* y1, const float* y2, const void* embed, const int* tokens,
+                 int embed_mode, float embed_scale, const void* w1, const void* w2, float offset, int T, int W, int V, float eps,
+                 int dtype, umb_stream_t stream);
+/* buf[i] *= scale, i < n */
+int umb_seq_scale(float* buf, long n, float scale, umb_stream_t stream);
+
+/* ---- rotary positions on a run of heads: in fp32 [T][ld] holds `heads` heads of D; the first rot_dims features of every head
+ * turn by pos * freq[i] (layout 0: feature i pairs with i + rot_dims / 2; 1: feature 2i with 2i + 1), the rest pass; the first
+ * heads_a heads are then multiplied by scale_a, the others by scale_b.  out fp32 [T][ldo]. */
+int umb_rope_scale(float* out, int ldo, const float* in, int ld, const int* pos, const float* freq, int T, int heads, int D,
+                   int rot_dims, int layout, int heads_a, float scale_a, float scale_b, umb_stream_t stream);
+/* alpha[t][h] = decay[h], log_alpha[t][h] = log(decay[h]) (log_alpha may be null): the rows the linear scans read */
+int umb_decay_fill(float* alpha, float* log_alpha, const float* decay, int T, int H, umb_stream_t stream);
+/* Behind a linear scan: o fp32 [T][H][P_cols], the head's Dv read-outs first.  den_col >= 0: column den_col holds n . q and the
+ * read-outs are divided by max(|n . q|, exp(-mrun[t][h])) + 1e-6 first.  Then each head over its root mean square (eps), times
+ * w ([Dv] shared by the heads, [H Dv] with w_per_head, or null), times silu (gate_kind 0) or sigmoid (1) of
+ * proj[t][g_col + h Dv + i], times out_scale, in `dtype` at out[t ldo + h Dv + i]. */
+int umb_head_gate(void* out, int ldo, const float* o, int P_cols, int den_col, const float* mrun, const float* proj, int ld,
+                  int g_col, const void* w, int w_per_head, int gate_kind, int T, int H, int Dv, float eps, float out_scale,
+                  int dtype, umb_stream_t stream);
+
+/* ---- softmax attention behind a short causal convolution.  proj fp32 [T][ld] = [q (H D) | k (G D) | v (G E) | ...] (biases
+ * added): every channel passes u_t = sum_j w[c][j] raw_(t - taps + 1 + j) (conv_w [C][taps] in `dtype`, null: none; earlier
+ * steps' inputs from conv_state fp32 [slots][taps - 1][C], position p in row p % (taps - 1)); q and k are RMS-normed over their
+ * WHOLE rows (weights w_q [H D], w_k [G D], null: 1) and rotated (rot_dims, layout and freq as umb_rope_scale); q -> fp32
+ * [T][H D], k and v -> the paged store.  The ring is refreshed by umb_ssd_conv_update (col0 0) afterwards, or here with
+ * update_state (steps of ONE token per sequence only).  The attention is umb_bsa_attend with a softcap. */
+int umb_cva_prep(float* q, const UmbPagedKV* kv, const float* proj, int ld, const void* conv_w, float* conv_state, const void* w_q,
+                 const void* w_k, const int* pos, const int* slot, const float* freq, int T, int H, int G, int D, int E, int taps,
+                 int rot_dims, int layout, int update_state, float eps, int dtype, umb_stream_t stream);
+
+/* ---- matrix memory with exponential gates.  gates fp32 [T][2 H] = [i | f]: i = cap tanh(z_i / cap), f = log sigmoid(cap
+ * tanh(z_f / cap)) from columns i_col / f_col of proj.  mscan: m_t = max(f_t + m_(t-1), i_t) token by token per (sequence, head)
+ * (mstate fp32 [slots][H]; a sequence that starts at position 0 starts from m = 0); log_alpha[t][h] = f_t + m_(t-1) - m_t, alpha
+ * its exponential, mrun[t][h] = m_t.  prep: qs fp32 [T][H D] = q * qscale; vp fp32 [T][H][Pp] = [e^(i - m) v | e^(i - m) | 0 ..]
+ * (Pp > Dv): a linear scan over (qs, k, vp, alpha) carries the matrix state and, as value column Dv, the normaliser.
+ * step: all three for steps of one token per sequence. */
+int umb_mlstm_gates(float* gates, const float* proj, int ld, int i_col, int f_col, int T, int H, float cap, umb_stream_t stream);
+int umb_mlstm_mscan(float* log_alpha, float* alpha, float* mrun, float* mstate, const float* gates, const int* seq_slot,
+                    const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int H, umb_stream_t stream);
+int umb_mlstm_prep(float* qs, float* vp, const float* proj, int ld, int q_col, int v_col, const float* gates, const float* mrun,
+                   int T, int H, int D, int Dv, int Pp, float qscale, umb_stream_t stream);
+int umb_mlstm_step(float* qs, float* vp, float* log_alpha, float* alpha, float* mrun, float* mstate, const float* proj, int ld,
+                   int q_col, int v_col, int i_col, int f_col, const int* pos, const int* slot, int T, int H, int D, int Dv, int Pp,
+                   float qscale, float cap, umb_stream_t stream);
+
+/* ---- routed experts chosen on the logits: the `top` largest of logits[t ld ..E] (ties: the lower index); wt = softmax over
+ * the chosen logits alone */
+int umb_moe_route_top(int* sel, float* wt, const float* logits, int ld, int T, int E, int top, umb_stream_t stream);
+/* y[t] = sigmoid(gate[t ldg]) * ys[t] + sum_k wt[t top + k] * ye[pos_of[t top + k]]  (ys null: none; gate null: 1; y may be ys) */
+int umb_moe_combine_gated(float* y, const float* ys, const float* ye, const float* wt, const int* pos_of, const float* gate,
+                          int ldg, int T, int W, int top, umb_stream_t stream);
 
 /* ------------------------------------------------------------------ the model */
 typedef struct UmbSeqLayer {
@@ -329,6 +402,29 @@ typedef struct UmbSeqLayer {
   const void *s_conv, *s_conv_b, *s_norm;
   const float *s_dt_bias, *s_a_log, *s_d;
   float* s_conv_state;        /* [slots][s_taps - 1][channels] fp32 */
+  /* retention (kind 5): proj = [q | k | v | g], heads x dim (q, k) and heads x vdim (v, g); decay fp32 [heads], one fixed decay
+   * per head; rotary (rot_layout 0: halves, 1: interleaved; rot_dims, rot_freq) on q and k, k times qscale after it; each head's
+   * read-out over its root mean square, times silu(g); state [slots][heads][dim][vdim].
+   * convolved attention beside a matrix memory (kind 6), both reading the same input: proj = [q | k | v | mq | mk | mv | mg | i | f];
+   * attention: heads / kv_heads / dim / vdim / scale / softcap, c_taps-tap convolution c_conv [(heads + kv_heads) dim + kv_heads
+   * vdim][c_taps] with ring c_conv_state, whole-row norms q_norm [heads dim] / k_norm [kv_heads dim], rotary as above; memory:
+   * m_heads x m_dim keys, m_vdim values, gates capped at gate_cap, m_norm [m_heads m_vdim], state [slots][m_heads][m_dim][m_pad]
+   * (value column m_vdim carries the normaliser) and the running maximum m_max [slots][m_heads]; the output projection reads
+   * [mix_scale_a * attention | mix_scale_b * memory] */
+  const float* decay;
+  int32_t rot_layout, c_taps;
+  float softcap, gate_cap;
+  const void* c_conv;
+  float* c_conv_state;
+  int32_t m_heads, m_dim, m_vdim, m_pad;
+  const void* m_norm;
+  float* m_max;
+  /* UMB_ACT_CLAMP_GLU: limits of the experts (or the dense feed-forward) and of the shared expert, the sigmoid's factor;
+   * shared_gate: the router's product has one more row, whose sigmoid multiplies the shared expert's output */
+  float act_limit, shared_limit, act_alpha;
+  int32_t shared_gate;
+  /* the embedding row is added to x once more right before this layer (a span of layers that runs again) */
+  int32_t add_embed, pad4_;
 } UmbSeqLayer;
 
 typedef struct UmbSeqModel {
@@ -339,8 +435,9 @@ typedef struct UmbSeqModel {
   /* streams >= 1: the residual is `streams` copies per token (ws.x is [Tmax][streams][W]), a sublayer is
    * x <- mix x + resid_mult * out * f(norm(in . x)) with norm weights stored around norm_offset, and the model ends with
    * the norm of the sum of the streams; 0: the single-stream forms above */
-  int32_t streams, pad_;
+  int32_t streams, block;    /* block: UMB_BLOCK_* (parallel: norms stored around norm_offset, ws.h2 / ws.y2 in use) */
   float resid_mult, norm_offset;
+  float logit_scale, pad2_;  /* the logits are multiplied by it (0 or 1: as they are) */
 } UmbSeqModel;
 
 /* activations of one step (caller-owned, sized for Tmax rows) */
@@ -365,6 +462,8 @@ typedef struct UmbSeqWork {
   float* moe_y;       /* [pairs][W] fp32 */
   int64_t moe_max_tiles;
   int64_t aux_floats;  /* floats in aux (what a step does not use of it serves as scratch) */
+  void* h2;            /* parallel blocks: normed input of the feed-forward [Tmax][W] dtype */
+  float* y2;           /* parallel blocks: feed-forward output [Tmax][W] fp32 */
 } UmbSeqWork;
 
 typedef struct UmbSeqStep {

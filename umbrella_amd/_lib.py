@@ -235,14 +235,21 @@ class UmbSeqLayer(C.Structure):
                 ("s_heads", C.c_int32), ("s_vdim", C.c_int32), ("s_state", C.c_int32), ("s_groups", C.c_int32),
                 ("s_norm_groups", C.c_int32), ("s_taps", C.c_int32),
                 ("s_conv", C.c_void_p), ("s_conv_b", C.c_void_p), ("s_norm", C.c_void_p),
-                ("s_dt_bias", C.c_void_p), ("s_a_log", C.c_void_p), ("s_d", C.c_void_p), ("s_conv_state", C.c_void_p)]
+                ("s_dt_bias", C.c_void_p), ("s_a_log", C.c_void_p), ("s_d", C.c_void_p), ("s_conv_state", C.c_void_p),
+                ("decay", C.c_void_p), ("rot_layout", C.c_int32), ("c_taps", C.c_int32),
+                ("softcap", C.c_float), ("gate_cap", C.c_float), ("c_conv", C.c_void_p), ("c_conv_state", C.c_void_p),
+                ("m_heads", C.c_int32), ("m_dim", C.c_int32), ("m_vdim", C.c_int32), ("m_pad", C.c_int32),
+                ("m_norm", C.c_void_p), ("m_max", C.c_void_p),
+                ("act_limit", C.c_float), ("shared_limit", C.c_float), ("act_alpha", C.c_float), ("shared_gate", C.c_int32),
+                ("add_embed", C.c_int32), ("pad4_", C.c_int32)]
 
 
 class UmbSeqModel(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("L", C.c_int32), ("W", C.c_int32), ("V", C.c_int32), ("groups", C.c_int32),
                 ("canon_taps", C.c_int32), ("eps", C.c_float), ("embed_scale", C.c_float), ("embed", C.c_void_p),
                 ("final_norm", C.c_void_p), ("head", UmbSeqLinear), ("layers", C.POINTER(UmbSeqLayer)),
-                ("streams", C.c_int32), ("pad_", C.c_int32), ("resid_mult", C.c_float), ("norm_offset", C.c_float)]
+                ("streams", C.c_int32), ("block", C.c_int32), ("resid_mult", C.c_float), ("norm_offset", C.c_float),
+                ("logit_scale", C.c_float), ("pad2_", C.c_float)]
 
 
 class UmbSeqWork(C.Structure):
@@ -250,7 +257,8 @@ class UmbSeqWork(C.Structure):
                 ("mix", C.c_void_p), ("act", C.c_void_p), ("y", C.c_void_p), ("logits", C.c_void_p),
                 ("Tmax", C.c_int32), ("Rmax", C.c_int32), ("moe_sel", C.c_void_p), ("moe_wt", C.c_void_p),
                 ("moe_pos", C.c_void_p), ("moe_tiles", C.c_void_p), ("moe_xs", C.c_void_p), ("moe_act", C.c_void_p),
-                ("moe_y", C.c_void_p), ("moe_max_tiles", C.c_int64), ("aux_floats", C.c_int64)]
+                ("moe_y", C.c_void_p), ("moe_max_tiles", C.c_int64), ("aux_floats", C.c_int64),
+                ("h2", C.c_void_p), ("y2", C.c_void_p)]
 
 
 class UmbSeqStep(C.Structure):
@@ -303,8 +311,22 @@ SEQ_SIGNATURES = {
     "umb_ssd_conv_update": [_P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I],
     "umb_ssd_gate": [_P, _I, _P, _P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I],
     "umb_bsa_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I],
-    "umb_bsa_attend": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P, _L, _I],
-    "umb_bsa_attend_tiled": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I],
+    "umb_bsa_attend": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P, _L, _I],
+    "umb_bsa_attend_tiled": [_P, _I, _P, _PKV, _P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _I],
+    "umb_seq_linear_glu": [_P, _P, _P, _P, _I, _I, _I, _F, _F, _I],
+    "umb_seq_linear_grouped_glu": [_P, _P, _P, _P, _I, _I, _L, _I, _I, _F, _F, _I],
+    "umb_blk_seam": [_P, _P, _P, _P, _P, _P, _P, _I, _F, _P, _P, _F, _I, _I, _I, _F, _I],
+    "umb_seq_scale": [_P, _L, _F],
+    "umb_rope_scale": [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F],
+    "umb_decay_fill": [_P, _P, _P, _I, _I],
+    "umb_head_gate": [_P, _I, _P, _I, _I, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _F, _I],
+    "umb_cva_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I],
+    "umb_mlstm_gates": [_P, _P, _I, _I, _I, _I, _I, _F],
+    "umb_mlstm_mscan": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I],
+    "umb_mlstm_prep": [_P, _P, _P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F],
+    "umb_mlstm_step": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _F],
+    "umb_moe_route_top": [_P, _P, _P, _I, _I, _I, _I],
+    "umb_moe_combine_gated": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I],
     "umb_bsa_attend_tiled_ok": [_I, _I, _I, _I, _I],
     "umb_moe_route_softmax": [_P, _P, _P, _P, _I, _I, _I],
     "umb_moe_combine_weighted": [_P, _P, _P, _P, _I, _I, _I, _I],

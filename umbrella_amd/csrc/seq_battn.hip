@@ -2,6 +2,7 @@
 //     q_i = unit_rms(W_q h_i) * w_q * temp(i)       k_j = unit_rms(W_k h_j) * w_k       v_j = unit_rms(W_v h_j)
 //     score(i, j, h) = q_i . k_j * scale + bias[h][min(i - j, n_dist - 1)]      (j <= i, i - j < window)
 //     out_i = c * sigmoid(gate_i[h]) * softmax_j(score) . v
+// With softcap > 0 the scaled product is capped before the bias joins it: softcap tanh(q . k scale / softcap).
 // temp(i) = 1 + coef ln(floor((i + 1) / every) + 1) sharpens the queries of long contexts; the bias table is indexed by the
 // clamped distance itself (whatever bucketing a design uses is expanded into it at load).  Keys and values are cached as
 // normed (storage dtype); queries, scores, weights, maxima and sums are fp32 (expf, not the fast intrinsic).
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(NW * 64) void bsa_attend_kernel(typename El<P>::typ
                                                              const float* __restrict__ bias, int n_dist,
                                                              const int* __restrict__ pos, const int* __restrict__ slot_, int H,
                                                              int G, int D, int E, int window, float scale, float out_scale,
-                                                             float* __restrict__ part, int nsplit) {
+                                                             float softcap, float* __restrict__ part, int nsplit) {
   typedef typename El<P>::type El_;
   extern __shared__ float lds[];
   constexpr int KB = 8;
@@ -135,7 +136,9 @@ __global__ __launch_bounds__(NW * 64) void bsa_attend_kernel(typename El<P>::typ
     const int bi = dist < n_dist ? dist : n_dist - 1;
 #pragma unroll
     for (int r = 0; r < RH; ++r) {
-      const float sv = kx < n_keys ? s[r] * scale + (bias ? bias[(long)(h0 + r) * n_dist + bi] : 0.f) : -INFINITY;
+      float sc = s[r] * scale;
+      if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);          // capped score; the bias (if any) is added to the capped value
+      const float sv = kx < n_keys ? sc + (bias ? bias[(long)(h0 + r) * n_dist + bi] : 0.f) : -INFINITY;
       const float m_new = fmaxf(m_run[r], wave_max(sv));          // finite: every round has at least one key
       const float fac = expf(m_run[r] - m_new);                   // 0 on the first round (m_run = -inf)
       const float pw = kx < n_keys ? expf(sv - m_new) : 0.f;
@@ -254,8 +257,8 @@ extern "C" int umb_bsa_prep(float* q, const UmbPagedKV* kv, const float* proj, i
 
 extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
                               const float* bias, int n_dist, const int* pos, const int* slot, int T, int H, int G, int D, int E,
-                              int window, float scale, float out_scale, float* scratch, long scratch_floats, int dtype,
-                              hipStream_t st) {
+                              int window, float scale, float out_scale, float softcap, float* scratch, long scratch_floats,
+                              int dtype, hipStream_t st) {
   if (T < 1 || H < 1 || G < 1 || H % G || D < 1 || E < 1 || E > 64 * BSA_MAXC || window < 1 || !out || !q || !bsa_kv_ok(kv) ||
       !pos || !slot || ldo < H * E || (bias && n_dist < 1) || (gate_col >= 0 && (!proj || ld < gate_col + H)))
     return UMB_EINVAL;
@@ -283,7 +286,7 @@ extern "C" int umb_bsa_attend(void* out, int ldo, const float* q, const UmbPaged
   do {                                                                                                                      \
     if (ensure_dynamic_lds<bsa_attend_kernel<P, RH, NC, NW>>(lds) != UMB_OK) return UMB_EHIP;                               \
     hipLaunchKernelGGL((bsa_attend_kernel<P, RH, NC, NW>), grid, dim3(NW * 64), lds, st, (El_*)out, ldo, q, *kv, proj, ld,  \
-                       gate_col, bias, n_dist, pos, slot, H, G, D, E, window, scale, out_scale, scratch, nsplit);           \
+                       gate_col, bias, n_dist, pos, slot, H, G, D, E, window, scale, out_scale, softcap, scratch, nsplit);           \
   } while (0)
 #define BSA_NW(RH, NC)                                                                                                      \
   if (nw == 16) BSA_LAUNCH(RH, NC, 16); else BSA_LAUNCH(RH, NC, 4)
@@ -330,7 +333,8 @@ __global__ __launch_bounds__(256) void bsa_attend_mfma_kernel(u16* __restrict__ 
                                                               const float* __restrict__ bias, int n_dist,
                                                               const int* __restrict__ seq_slot, const int* __restrict__ seq_row0,
                                                               const int* __restrict__ seq_pos0, const int* __restrict__ seq_len,
-                                                              int H, int G, int D, int E, int window, float scale, float out_scale) {
+                                                              int H, int G, int D, int E, int window, float scale, float out_scale,
+                                                              float softcap) {
   extern __shared__ __attribute__((aligned(16))) u16 bsa_lds[];
   constexpr int NLK = (NSM * 4 + 7) / 8, NLV = (NVM * 2 + 7) / 8;     // 16-byte chunks of a key / value row per staging thread
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g4 = lane >> 4;
@@ -470,7 +474,9 @@ __global__ __launch_bounds__(256) void bsa_attend_mfma_kernel(u16* __restrict__ 
       float sv[8], mx = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        sv[e] = vis[e] ? sc2[hh][e >> 2][e & 3] * scale2 + bv[hh][e] * BSA_LOG2E : -INFINITY;
+        float raw = sc2[hh][e >> 2][e & 3] * scale2;
+        if (softcap > 0.f) raw = softcap * tanhf(sc2[hh][e >> 2][e & 3] * scale / softcap) * BSA_LOG2E;      // capped, then to base 2
+        sv[e] = vis[e] ? raw + bv[hh][e] * BSA_LOG2E : -INFINITY;
         mx = fmaxf(mx, sv[e]);
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -542,7 +548,7 @@ extern "C" int umb_bsa_attend_tiled_ok(int H, int G, int D, int E, int dtype) {
 extern "C" int umb_bsa_attend_tiled(void* out, int ldo, const float* q, const UmbPagedKV* kv, const float* proj, int ld,
                                     int gate_col, const float* bias, int n_dist, const int* seq_slot, const int* seq_row0,
                                     const int* seq_pos0, const int* seq_len, int B, int max_len, int H, int G, int D, int E,
-                                    int window, float scale, float out_scale, int dtype, hipStream_t st) {
+                                    int window, float scale, float out_scale, float softcap, int dtype, hipStream_t st) {
   if (B < 1 || B > 65535 || max_len < 1 || window < 1 || !out || !q || !bsa_kv_ok(kv) || !seq_slot || !seq_row0 || !seq_pos0 ||
       !seq_len || ldo < H * E || (bias && n_dist < 1) || (gate_col >= 0 && (!proj || ld < gate_col + H)) ||
       !umb_bsa_attend_tiled_ok(H, G, D, E, dtype))
@@ -558,7 +564,7 @@ extern "C" int umb_bsa_attend_tiled(void* out, int ldo, const float* q, const Um
     if (ensure_dynamic_lds<bsa_attend_mfma_kernel<P, NSM, NVM, HPW>>(lds) != UMB_OK) return UMB_EHIP;                      \
     hipLaunchKernelGGL((bsa_attend_mfma_kernel<P, NSM, NVM, HPW>), grid, dim3(256), lds, st, (u16*)out, ldo, q, *kv, proj, \
                        ld, gate_col, bias, n_dist, seq_slot, seq_row0, seq_pos0, seq_len, H, G, D, E, window, scale,       \
-                       out_scale);                                                                                         \
+                       out_scale, softcap);                                                                                \
   } while (0)
 #define BSA_MFMA_SHAPE()                                                                                                   \
   if (D <= 128 && E <= 128) { if (hpg > 4) BSA_MFMA(4, 8, 2); else BSA_MFMA(4, 8, 1); }                                    \

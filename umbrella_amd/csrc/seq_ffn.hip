@@ -253,3 +253,68 @@ extern "C" int umb_moe_combine_weighted(float* y, const float* ye, const float* 
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }
+
+// Routing on the logits themselves: the `top` largest logits of a token (ties: the lower index) are chosen and their weights are
+// the softmax over JUST the chosen logits (fp32, expf).  logits rows are ld apart (other columns may follow the E logits).
+__global__ __launch_bounds__(256) void moe_route_top_kernel(int* __restrict__ sel, float* __restrict__ wt,
+                                                            const float* __restrict__ logits, int ld, int T, int E, int top) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  const float* z = logits + (long)t * ld;
+  int prev_i = -1;
+  float prev_z = INFINITY, first = 0.f, tot = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = z[e];
+      const bool after = v < prev_z || (v == prev_z && e > prev_i);
+      if (after && (v > best || (v == best && e < bi))) { best = v; bi = e; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    if (bi >= E) { bi = 0; best = -INFINITY; }      // no candidate left (logits that are not numbers): keep indices in range
+    if (k == 0) first = best;                       // the largest logit: every exponent below is <= 0
+    const float ev = expf(best - first);
+    tot += ev;
+    if (lane == 0) { sel[(long)t * top + k] = bi; wt[(long)t * top + k] = ev; }
+    prev_z = best; prev_i = bi;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) wt[(long)t * top + k] = wt[(long)t * top + k] / tot;
+}
+
+// y[t] = sigmoid(gate[t ldg]) * ys[t] + sum_k wt[t top + k] * ye[pos_of[t top + k]]   (ys null: no shared part; gate null: 1)
+__global__ __launch_bounds__(256) void moe_combine_gated_kernel(float* y, const float* ys, const float* __restrict__ ye,
+                                                                const float* __restrict__ wt, const int* __restrict__ pos_of,
+                                                                const float* __restrict__ gate, int ldg, int W, int top) {
+  const int t = blockIdx.x;
+  const float gs = gate ? 1.f / (1.f + expf(-gate[(long)t * ldg])) : 1.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float a = 0.f;
+    for (int k = 0; k < top; ++k) a += wt[(long)t * top + k] * ye[(long)pos_of[(long)t * top + k] * W + c];
+    y[(long)t * W + c] = ys ? a + gs * ys[(long)t * W + c] : a;
+  }
+}
+
+extern "C" int umb_moe_route_top(int* sel, float* wt, const float* logits, int ld, int T, int E, int top, hipStream_t st) {
+  if (T < 1 || E < 1 || top < 1 || top > E || ld < E || !sel || !wt || !logits) return UMB_EINVAL;
+  hipLaunchKernelGGL(moe_route_top_kernel, dim3((T + 3) / 4), dim3(256), 0, st, sel, wt, logits, ld, T, E, top);
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_moe_combine_gated(float* y, const float* ys, const float* ye, const float* wt, const int* pos_of,
+                                     const float* gate, int ldg, int T, int W, int top, hipStream_t st) {
+  if (T < 1 || W < 1 || top < 1 || !y || !ye || !wt || !pos_of) return UMB_EINVAL;
+  hipLaunchKernelGGL(moe_combine_gated_kernel, dim3(T), dim3(256), 0, st, y, ys, ye, wt, pos_of, gate, ldg, W, top);
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}

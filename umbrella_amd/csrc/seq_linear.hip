@@ -56,7 +56,18 @@ template <> __device__ __forceinline__ f32x4 mma8<F32>(const Frag8<F32>& a, cons
   return c;
 }
 
-enum { EPI_F32 = 0, EPI_DT = 1, EPI_SILU_MUL = 2, EPI_GATE = 3, EPI_RELU2 = 4 };
+enum { EPI_F32 = 0, EPI_DT = 1, EPI_SILU_MUL = 2, EPI_GATE = 3, EPI_RELU2 = 4, EPI_CLAMP_GLU = 5 };
+// the two stacked-halves epilogues: silu(gate) * up, or the capped form g sigmoid(alpha g) (u + 1) with g = min(gate, limit),
+// u = clamp(up, -limit, limit)
+static inline bool epi_dual(int epi) { return epi == EPI_SILU_MUL || epi == EPI_CLAMP_GLU; }
+__device__ __forceinline__ float glu_pair(int epi, float g, float u, float limit, float alpha) {
+  if (epi == EPI_CLAMP_GLU) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+  }
+  return siluf_(g) * u;
+}
 
 // Where a launch departs from the dense [T][K] x [N][K] problem: row strides of x and out, a batch of independent problems
 // along blockIdx.z (element strides sx / sw / so), or token tiles read from device memory (grouped: tile blockIdx.y is
@@ -67,6 +78,7 @@ struct LinExt {
   const int* tiles;
   const float* gate;
   int ldg, sg;
+  float limit, alpha;      // EPI_CLAMP_GLU
 };
 static inline LinExt lin_dense(int N, int K) { return LinExt{K, N, 0, 0, 0, 0, nullptr, nullptr, 0, 0}; }
 
@@ -181,7 +193,7 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
 #pragma unroll
         for (int ww = 1; ww < 4; ++ww) u += red[1][ww][nt * TT + tt][threadIdx.x];
         u += bv2;
-        stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, siluf_(s) * u);
+        stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, glu_pair(epi, s, u, ext.limit, ext.alpha));
       } else if (epi == EPI_DT) {
         stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, s);
       } else if (epi == EPI_RELU2) {
@@ -301,7 +313,7 @@ __global__ __launch_bounds__(256) void seq_linear_wide_kernel(void* __restrict__
         float sv = acc[i][tt][r] + (bias ? P::to_f(bias[n]) : 0.f);
         if constexpr (DUAL) {
           const float uv = acc[i + 2][tt][r] + (bias ? P::to_f(bias[N + n]) : 0.f);
-          reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(siluf_(sv) * uv);
+          reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(glu_pair(epi, sv, uv, ext.limit, ext.alpha));
         } else if (epi == EPI_DT) {
           reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(sv);
         } else if (epi == EPI_RELU2) {
@@ -320,7 +332,7 @@ static int launch_wide(void* out, const void* x, const void* w, const void* bias
                        const LinExt& ext = LinExt{0, 0, 0, 0, 0, 0, nullptr, nullptr, 0, 0}, int gy = 0) {
   if constexpr (sizeof(typename El<P>::type) == 2) {
     const unsigned ty = gy > 0 ? gy : (T + 127) / 128;
-    if (epi == EPI_SILU_MUL)
+    if (epi_dual(epi))
       hipLaunchKernelGGL((seq_linear_wide_kernel<P, true>), dim3((N + 63) / 64, ty), dim3(256), 0, st, out,
                          (const u16*)x, (const u16*)w, (const u16*)bias, T, N, K, epi, ext);
     else
@@ -340,7 +352,7 @@ static int launch_tt(void* out, const void* x, const void* w, const void* bias, 
   typedef typename El<P>::type E;
   constexpr int NTD = NT > 2 ? 2 : NT;             // gate/up: two tile pairs at most
   const dim3 grid((N + NT * 16 - 1) / (NT * 16), gy > 0 ? gy : (T + TT * 16 - 1) / (TT * 16), gz);
-  if (epi == EPI_SILU_MUL)
+  if (epi_dual(epi))
     hipLaunchKernelGGL((seq_linear_kernel<P, NTD, TT, VEC, true>), dim3((N + NTD * 16 - 1) / (NTD * 16), grid.y, gz), dim3(256), 0,
                        st, out, (const E*)x, (const E*)w, (const E*)bias, T, N, K, epi, ext);
   else
@@ -359,24 +371,38 @@ static int launch_vec(void* out, const void* x, const void* w, const void* bias,
   // (the K order of every output is unchanged: a row's value does not depend on which variant computed it)
   const bool dense = gz == 1 && ext.ldx == K && ext.ldo == N && epi != EPI_GATE;
   if (T > 64 && N >= 64 && sizeof(typename El<P>::type) == 2) {
-    if (VEC && dense && T >= 256 && N >= 128) return launch_wide<P>(out, x, w, bias, T, N, K, epi, st);      // both operands re-used
+    if (VEC && dense && T >= 256 && N >= 128) return launch_wide<P>(out, x, w, bias, T, N, K, epi, st, LinExt{0, 0, 0, 0, 0, 0, nullptr, nullptr, 0, 0, ext.limit, ext.alpha});      // both operands re-used
     return launch_tt<P, 4, 4, VEC>(out, x, w, bias, T, N, K, epi, st, ext, 0, gz);
   }
   return launch_tt<P, 1, 4, VEC>(out, x, w, bias, T, N, K, epi, st, ext, 0, gz);
 }
 
-extern "C" int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, int dtype,
-                              hipStream_t st) {
-  if (T < 1 || N < 1 || K < 1 || epi < 0 || (epi > 2 && epi != EPI_RELU2) || !out || !x || !w) return UMB_EINVAL;
-  if (epi == EPI_SILU_MUL) {
+static int seq_linear_any(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, float limit,
+                          float alpha, int dtype, hipStream_t st) {
+  if (T < 1 || N < 1 || K < 1 || epi < 0 || (epi > 2 && epi != EPI_RELU2 && epi != EPI_CLAMP_GLU) || !out || !x || !w) return UMB_EINVAL;
+  if (epi_dual(epi)) {
     if (N & 1) return UMB_EINVAL;
     N >>= 1;                                   // rows of each half
   }
-  const LinExt ext = lin_dense(N, K);
+  LinExt ext = lin_dense(N, K);
+  ext.limit = limit;
+  ext.alpha = alpha;
   DISPATCH_SEQ_DTYPE(dtype, {
     if (K % 8 == 0) return launch_vec<P, true>(out, x, w, bias, T, N, K, epi, st, ext);
     return launch_vec<P, false>(out, x, w, bias, T, N, K, epi, st, ext);
   })
+}
+
+extern "C" int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, int dtype,
+                              hipStream_t st) {
+  if (epi == EPI_CLAMP_GLU) return UMB_EINVAL;              // that epilogue has constants: umb_seq_linear_glu
+  return seq_linear_any(out, x, w, bias, T, N, K, epi, 0.f, 0.f, dtype, st);
+}
+
+extern "C" int umb_seq_linear_glu(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, float limit,
+                                  float alpha, int dtype, hipStream_t st) {
+  if (!(limit > 0.f)) return UMB_EINVAL;
+  return seq_linear_any(out, x, w, bias, T, N, K, EPI_CLAMP_GLU, limit, alpha, dtype, st);
 }
 
 extern "C" int umb_seq_linear_batched(void* out, const void* x, const void* w, int T, int N, int K, int ldx, int ldo, int batch,
@@ -394,16 +420,17 @@ extern "C" int umb_seq_linear_batched(void* out, const void* x, const void* w, i
   })
 }
 
-extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows,
-                                      long gs, int N, int K, int epi, int dtype, hipStream_t st) {
-  if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || (epi > 2 && epi != EPI_RELU2) || !out || !x || !w || !tiles ||
+static int seq_linear_grouped_any(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows, long gs,
+                                  int N, int K, int epi, float limit, float alpha, int dtype, hipStream_t st) {
+  if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || (epi > 2 && epi != EPI_RELU2 && epi != EPI_CLAMP_GLU) || !out ||
+      !x || !w || !tiles ||
       (tile_rows != 16 && tile_rows != 64 && tile_rows != 128))
     return UMB_EINVAL;
-  if (epi == EPI_SILU_MUL) {
+  if (epi_dual(epi)) {
     if (N & 1) return UMB_EINVAL;
     N >>= 1;
   }
-  const LinExt ext{K, N, 0, 0, 0, gs, tiles, nullptr, 0, 0};
+  const LinExt ext{K, N, 0, 0, 0, gs, tiles, nullptr, 0, 0, limit, alpha};
   if (tile_rows == 128) {                  // many rows per group: both operands staged through LDS (16-bit storage only)
     if (dtype == UMB_SEQ_F32 || K % 8 || gs % 8) return UMB_EINVAL;
     if (dtype == UMB_SEQ_BF16) return launch_wide<BF16>(out, x, w, nullptr, 128, N, K, epi, st, ext, max_tiles);
@@ -422,4 +449,16 @@ extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, c
     }
     return launch_tt<P, 1, 4, false>(out, x, w, nullptr, 64, N, K, epi, st, ext, max_tiles);
   })
+}
+
+extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows,
+                                      long gs, int N, int K, int epi, int dtype, hipStream_t st) {
+  if (epi == EPI_CLAMP_GLU) return UMB_EINVAL;
+  return seq_linear_grouped_any(out, x, w, tiles, max_tiles, tile_rows, gs, N, K, epi, 0.f, 0.f, dtype, st);
+}
+
+extern "C" int umb_seq_linear_grouped_glu(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows,
+                                          long gs, int N, int K, float limit, float alpha, int dtype, hipStream_t st) {
+  if (!(limit > 0.f)) return UMB_EINVAL;
+  return seq_linear_grouped_any(out, x, w, tiles, max_tiles, tile_rows, gs, N, K, EPI_CLAMP_GLU, limit, alpha, dtype, st);
 }

@@ -16,12 +16,13 @@ from .fidizen import Fidizen
 from .gitopel import Gitopel
 from .llama import Llama
 from .tomopel import Tomopel
+from .zusuvik import Zusuvik
 
 
 class AutoModelLM:
     # a local directory is resolved by the architecture its config.json names; directories that name none of these are
     # Hugging Face Llama / Qwen2 / Mistral checkpoints
-    _ARCHITECTURE_MAPPING = {"Gitopel": Gitopel, "Fidizen": Fidizen, "Tomopel": Tomopel}
+    _ARCHITECTURE_MAPPING = {"Gitopel": Gitopel, "Fidizen": Fidizen, "Tomopel": Tomopel, "Zusuvik": Zusuvik}
     _MODEL_MAPPING = {name: Llama for name in KNOWN}
     _OFFLOAD_MODEL_MAPPING = dict(_MODEL_MAPPING)
     _CUDAGRAPH_MODEL_MAPPING = dict(_MODEL_MAPPING)

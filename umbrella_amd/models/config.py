@@ -284,9 +284,79 @@ class AttnSSDCfg:
     kind: str = "attention_ssd"
 
 
+def rotary_frequencies(base: float, dims: int, scaling: Optional[dict] = None) -> torch.Tensor:
+    """fp32 [dims / 2]: f_i = base^(-2 i / dims), formed in float64 and rounded once.  ``scaling`` = {factor, low, high,
+    original} slows the long wavelengths: with l = 2 pi / f, f stays where l < original / high, becomes f / factor where
+    l > original / low, and is blended in between with s = (original / l - low) / (high - low): (1 - s) f / factor + s f."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    if scaling:
+        factor, low, high = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+        orig = float(scaling["original"])
+        wl = 2.0 * math.pi / f
+        s = (orig / wl - low) / (high - low)
+        blend = (1.0 - s) * f / factor + s * f
+        f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, blend))
+    return f.to(torch.float32)
+
+
+@dataclass
+class RetentionCfg:
+    """Linear attention with one FIXED decay per head (``decay``: a number per head) and neither softmax nor denominator:
+    per-head [dim, vdim] fp32 state; rotary positions on the first ``rot_dims`` features of q and k (``rot_layout`` 'half':
+    feature i pairs with i + rot_dims / 2; 'interleaved': 2i with 2i + 1), k times dim^-1/2 after it; each head's read-out over
+    its root mean square, times silu of a gate projection."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: list
+    rot_dims: int
+    rot_base: float
+    rot_scaling: Optional[dict] = None
+    rot_layout: str = "half"
+    kind: str = "retention"
+
+
+@dataclass
+class AttnMLSTMCfg:
+    """Two mixers side by side that read the same input and share one output projection over ``[a_scale * attention |
+    b_scale * memory]``.
+
+    Attention: causal softmax, grouped query heads, projections with biases; q, k and v first pass a causal convolution of
+    ``taps`` taps per channel (its last inputs are state), q and k an RMS norm over the WHOLE projection (plain weights), then
+    rotary positions (``rot_*`` as in ``RetentionCfg``, frequencies optionally scaled); scores are capped:
+    ``softcap tanh(q . k scale / softcap)`` (0: not capped).
+    Memory: ``m_heads`` heads with a ``[m_dim, m_vdim]`` fp32 matrix state, a normaliser and a running maximum each;
+    exponential input / forget gates capped at ``gate_cap``; per-head unit RMS, a weight over all heads, a sigmoid gate."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float
+    taps: int
+    rot_dims: int
+    rot_base: float
+    rot_scaling: Optional[dict]
+    a_scale: float
+    m_heads: int
+    m_dim: int
+    m_vdim: int
+    gate_cap: float
+    b_scale: float
+    rot_layout: str = "interleaved"
+    window: int = 0
+    kind: str = "attention_mlstm"
+
+    @property
+    def m_pad(self) -> int:
+        """value columns of the carried state: the values, the normaliser's column, up to a multiple of four"""
+        return (self.m_vdim + 1 + 3) // 4 * 4
+
+
 @dataclass
 class SeqLayerCfg:
-    mixer: object                    # PooledWindowAttnCfg | GLACfg | LatentAttnCfg | MinGRUCfg | AttnSSDCfg
+    mixer: object                    # PooledWindowAttnCfg | GLACfg | LatentAttnCfg | MinGRUCfg | AttnSSDCfg | RetentionCfg | AttnMLSTMCfg
     ff: int = 0                      # width of the dense feed-forward; 0 = the layer has none (or has experts)
     ff_kind: str = "gated"           # "gated": W_down (silu(W_gate h) * W_up h); "polynorm": W_down polynorm(W_up h); "moe"
     experts: int = 0                 # "moe": routed experts, how many each token uses, their width, the shared expert's
@@ -296,7 +366,16 @@ class SeqLayerCfg:
     weights_of: int | None = None    # the layer uses that layer's tensors (with a cache and state of its own)
     act: str = "silu_gated"          # "silu_gated": silu(W_gate h) * W_up h; "relu2": relu(W_up h)^2 (no gate) -- dense, experts, shared
     route: str = "sigmoid_in"        # "sigmoid_in": sigmoid scores weigh the expert's input; "softmax_out": softmax scores,
-                                     # chosen with a correction added, renormalised over the chosen, weigh its output
+                                     # chosen with a correction added, renormalised over the chosen, weigh its output;
+                                     # "top_logits": the largest logits, softmax over the chosen alone, weigh its output
+    # act "clamp_glu": g sigmoid(act_alpha g) (u + 1) with g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit); the
+    # limit of the experts / the dense feed-forward and the shared expert's own
+    act_limit: float = 0.0
+    shared_limit: float = 0.0
+    act_alpha: float = 1.702
+    shared_gate: bool = False        # the shared expert's output is multiplied by sigmoid(w . h), one number per token
+    add_embed: bool = False          # the embedding row is added to the residual once more right before this layer
+    tensor_prefix: str = ""          # checkpoint prefix of the layer's tensors where it is not "l<index>."
 
     @property
     def has_ff(self) -> bool:
@@ -319,7 +398,9 @@ class SeqMixCfg:
     streams: int = 0                 # >= 1: that many residual streams with read / write / mix weights per sublayer (norms
                                      # in front of the sublayers only); 0: one stream with the seams above
     resid_mult: float = 1.0          # a sublayer's output is multiplied by it before it joins the residual (streams >= 1)
-    norm_offset: float = 0.0         # norm weights are stored around it: the factor is offset + w (streams >= 1)
+    norm_offset: float = 0.0         # norm weights are stored around it: the factor is offset + w (streams >= 1, parallel blocks)
+    block: str = "sequential"        # "parallel": both sublayers of a layer read the same residual, x + (mixer(norm1 x) + ff(norm2 x))
+    logit_scale: float = 1.0         # the logits are multiplied by it
 
     @property
     def num_hidden_layers(self):

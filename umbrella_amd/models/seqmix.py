@@ -1,11 +1,12 @@
 """Runtime of the sequence-mixer model family on the HIP path (libumbrella_seq.so, include/umbrella_seq.h).
 
 A model is a LIST of layers, each a token mixer -- windowed attention with pooled blocks, gated linear attention, latent
-attention, a minimal gated recurrence, or softmax attention beside a state-space layer -- plus an optional feed-forward (gated
-SiLU, PolyNorm, or routed experts with a shared one).  A sublayer reads either a grouped RMS norm of the residual stream or the
+attention, a minimal gated recurrence, softmax attention beside a state-space layer, retention, or convolved softmax
+attention beside a matrix memory -- plus an optional feed-forward (gated SiLU, PolyNorm, or routed experts with a shared one).  A sublayer reads either a grouped RMS norm of the residual stream or the
 stream itself through a short causal convolution; its output is normed before it is added back; or (``streams >= 1``) the
 residual is several streams that every sublayer reads as one combination and writes back to all.  A layer may use another
-layer's tensors with a cache and state of its own.  The list, every size and every
+layer's tensors with a cache and state of its own; or (``block == "parallel"``) both sublayers of a layer read the same
+residual and their outputs are added to it together.  The list, every size and every
 constant come from a ``SeqMixCfg`` (models/config.py); a design contributes a subclass that names its checkpoint tensors
 (models/gitopel.py, models/fidizen.py).
 
@@ -27,12 +28,15 @@ from .. import _lib
 from .._lib import UmbSeqLayer, UmbSeqLinear, UmbSeqModel, UmbSeqStep, UmbSeqWork
 from ..attn.cache import PagedSeqCache
 from .base import LLMBase
-from .config import SeqMixCfg
+from .config import SeqMixCfg, rotary_frequencies
 
-KIND_CODE = {"attention": 0, "gla": 1, "latent_attention": 2, "mingru": 3, "attention_ssd": 4}
+KIND_CODE = {"attention": 0, "gla": 1, "latent_attention": 2, "mingru": 3, "attention_ssd": 4, "retention": 5,
+             "attention_mlstm": 6}
 FF_CODE = {"gated": 0, "polynorm": 1, "moe": 2}
-ACT_CODE = {"silu_gated": 0, "relu2": 1}
-ROUTE_CODE = {"sigmoid_in": 0, "softmax_out": 1}
+ACT_CODE = {"silu_gated": 0, "relu2": 1, "clamp_glu": 2}
+ROUTE_CODE = {"sigmoid_in": 0, "softmax_out": 1, "top_logits": 2}
+BLOCK_CODE = {"sequential": 0, "parallel": 1}
+ROT_LAYOUT_CODE = {"half": 0, "interleaved": 1}
 
 
 def _linear(w, b=None) -> UmbSeqLinear:
@@ -138,12 +142,28 @@ class SeqMixLM(LLMBase):
                 kv_layers.append((m.kv_heads, m.dim, 0, m.vdim))
                 state_layers.append((m.s_heads, m.s_state, m.s_vdim))
                 mixer_convs.append((m.s_taps, m.s_heads * m.s_vdim + 2 * m.s_groups * m.s_state))
+            elif m.kind == "retention":
+                if len(m.decay) != m.heads:
+                    raise ValueError("retention wants one decay per head")
+                t["cache_index"] = len(state_layers)
+                state_layers.append((m.heads, m.dim, m.vdim))
+                t["decay"] = torch.tensor([float(d) for d in m.decay], dtype=torch.float32, device=dev)
+            elif m.kind == "attention_mlstm":
+                if m.heads % m.kv_heads:
+                    raise ValueError("heads must be a multiple of kv_heads")
+                t["cache_index"], t["state_index"], t["mconv_index"] = len(kv_layers), len(state_layers), len(mixer_convs)
+                kv_layers.append((m.kv_heads, m.dim, 0, m.vdim))
+                state_layers.append((m.m_heads, m.m_dim, m.m_pad))      # value column m_vdim carries the normaliser
+                state_layers.append((m.m_heads, 1, 1))                  # the running maximum
+                mixer_convs.append((m.taps, (m.heads + m.kv_heads) * m.dim + m.kv_heads * m.vdim))
             else:
                 t["cache_index"] = len(state_layers)
                 state_layers.append((m.heads, m.dim, m.vdim))
             if m.kind in ("attention", "latent_attention") and "rot_freq" not in t:
                 i2 = torch.arange(m.rot_dims // 2, dtype=torch.float32)
                 t["rot_freq"] = (m.rot_base ** (-2 * i2 / m.rot_dims)).to(dev) if m.rot_dims else None     # fp32 frequencies
+            if m.kind in ("retention", "attention_mlstm") and "rot_freq" not in t:
+                t["rot_freq"] = rotary_frequencies(m.rot_base, m.rot_dims, m.rot_scaling).to(dev) if m.rot_dims else None
             if c.canon_taps > 0:
                 t["conv_index"] = n_conv
                 n_conv += 2 if ly.has_ff else 1
@@ -197,10 +217,33 @@ class SeqMixLM(LLMBase):
                 s.s_conv_state = self.kv_cache.mixer_conv[t["mconv_index"]].data_ptr()
                 s.kv = self.kv_cache.struct(t["cache_index"])
                 s.state = self.kv_cache.state[t["state_index"]].data_ptr()
+            elif m.kind == "retention":
+                s.rot_dims, s.rot_layout, s.qscale = m.rot_dims, ROT_LAYOUT_CODE[m.rot_layout], float(m.dim) ** -0.5
+                s.rot_freq = t["rot_freq"].data_ptr() if t["rot_freq"] is not None else None
+                s.decay = t["decay"].data_ptr()
+                s.state = self.kv_cache.state[t["cache_index"]].data_ptr()
+            elif m.kind == "attention_mlstm":
+                s.kv_heads, s.scale, s.softcap = m.kv_heads, float(m.scale), float(m.softcap)
+                s.window = m.window if m.window > 0 else 2 ** 30
+                s.rot_dims, s.rot_layout = m.rot_dims, ROT_LAYOUT_CODE[m.rot_layout]
+                s.rot_freq = t["rot_freq"].data_ptr() if t["rot_freq"] is not None else None
+                s.q_norm = t["q_norm"].data_ptr() if t.get("q_norm") is not None else None
+                s.k_norm = t["k_norm"].data_ptr() if t.get("k_norm") is not None else None
+                s.c_taps = m.taps
+                s.c_conv = t["c_conv"].data_ptr() if t.get("c_conv") is not None else None
+                s.c_conv_state = self.kv_cache.mixer_conv[t["mconv_index"]].data_ptr()
+                s.mix_scale_a, s.mix_scale_b, s.gate_cap = float(m.a_scale), float(m.b_scale), float(m.gate_cap)
+                s.m_heads, s.m_dim, s.m_vdim, s.m_pad = m.m_heads, m.m_dim, m.m_vdim, m.m_pad
+                s.m_norm = t["m_norm"].data_ptr() if t.get("m_norm") is not None else None
+                s.kv = self.kv_cache.struct(t["cache_index"])
+                s.state = self.kv_cache.state[t["state_index"]].data_ptr()
+                s.m_max = self.kv_cache.state[t["state_index"] + 1].data_ptr()
             else:
                 s.rank, s.tau, s.qscale = m.rank, m.tau, float(m.dim) ** -0.5
                 s.a2, s.head_norm = _linear(t["a2_w"], t["a2_b"]), t["head_norm"].data_ptr()
                 s.state = self.kv_cache.state[t["cache_index"]].data_ptr()
+            s.add_embed = int(ly.add_embed)
+            s.act_limit, s.shared_limit, s.act_alpha = float(ly.act_limit), float(ly.shared_limit), float(ly.act_alpha)
             if ly.has_ff:
                 s.norm2 = t["norm2"].data_ptr() if t.get("norm2") is not None else None
                 s.norm2b = t["norm2b"].data_ptr() if t.get("norm2b") is not None else None
@@ -208,7 +251,8 @@ class SeqMixLM(LLMBase):
                     s.canon2, s.canon_state2 = t["canon2"].data_ptr(), self.kv_cache.conv[t["conv_index"] + 1].data_ptr()
                 if ly.ff_kind == "moe":
                     s.experts, s.top, s.expert_ff, s.shared_ff = ly.experts, ly.top, ly.expert_ff, ly.shared_ff
-                    s.router, s.e_gu, s.e_down = _linear(t["router_w"]), t["e_gu"].data_ptr(), t["e_down"].data_ptr()
+                    s.router, s.e_gu, s.e_down = _linear(t["router_w"], t.get("router_b")), t["e_gu"].data_ptr(), t["e_down"].data_ptr()
+                    s.shared_gate = int(ly.shared_gate)
                     s.correction = t["correction"].data_ptr() if t.get("correction") is not None else None
                     if ly.shared_ff:
                         s.s_gu, s.s_down = _linear(t["s_gu_w"]), _linear(t["s_down_w"])
@@ -220,6 +264,7 @@ class SeqMixLM(LLMBase):
         mdl.dtype, mdl.L, mdl.W, mdl.V, mdl.groups, mdl.eps = _lib.seq_dtype_code(dt), L, c.width, c.vocab_size, c.norm_groups, c.norm_eps
         mdl.embed_scale, mdl.canon_taps = float(c.embed_scale), int(c.canon_taps)
         mdl.streams, mdl.resid_mult, mdl.norm_offset = int(c.streams), float(c.resid_mult), float(c.norm_offset)
+        mdl.block, mdl.logit_scale = BLOCK_CODE[c.block], float(c.logit_scale)
         mdl.embed, mdl.final_norm, mdl.head = self._top["embed"].data_ptr(), self._top["final_norm"].data_ptr(), _linear(self._top["head"])
         mdl.layers = C.cast(self._layer_structs, C.POINTER(UmbSeqLayer))
         self.reserve(self.max_step_tokens or 256)
@@ -259,10 +304,20 @@ class SeqMixLM(LLMBase):
                 chunk = m.s_heads * (m.s_state * m.s_vdim + 1)
                 ask(aux=m.heads * m.dim + 2 * inner + 2 * m.s_groups * m.s_state + 2 * m.s_heads + (chunk + 63) // 64 + (8 * chunk) // T + 1,
                     o=inner, mix=m.heads * m.vdim + inner)
+            elif m.kind == "retention":
+                # aux: rotated [q | k] | decay rows and their logarithms | chunk states of the chunked scan
+                chunk = m.heads * (m.dim * m.vdim + 1)
+                ask(aux=2 * m.heads * m.dim + 2 * m.heads + (chunk + 63) // 64 + (8 * chunk + 64) // T + 1, o=m.heads * m.vdim,
+                    mix=m.heads * m.vdim)
+            elif m.kind == "attention_mlstm":
+                # aux: queries | scaled memory queries | widened values | gates, decays, logarithms, maxima | chunk states
+                chunk = m.m_heads * (m.m_dim * m.m_pad + 1)
+                ask(aux=m.heads * m.dim + m.m_heads * (m.m_dim + m.m_pad + 5) + (chunk + 63) // 64 + (8 * chunk + 64) // T + 1,
+                    o=m.m_heads * m.m_pad, mix=m.heads * m.vdim + m.m_heads * m.m_vdim)
             else:
                 ask(aux=m.heads * m.dim, o=m.heads * m.vdim, mix=m.heads * m.vdim)
             if ly.ff_kind == "moe":
-                ask(proj=ly.experts, act=ly.shared_ff)
+                ask(proj=ly.experts + 1, act=ly.shared_ff)
                 top, eff = max(top, ly.top), max(eff, ly.expert_ff)
             elif ly.ff:
                 ask(act=ly.ff, proj=ly.ff if ly.ff_kind == "polynorm" else 1)
@@ -276,6 +331,9 @@ class SeqMixLM(LLMBase):
         ws = self._ws = UmbSeqWork()
         for k in ("x", "h", "proj", "aux", "o", "mix", "act", "y", "logits"):
             setattr(ws, k, b[k].data_ptr())
+        if c.block == "parallel":                       # the feed-forward's own normed input and output
+            b.update(h2=torch.zeros(T, c.width, dtype=dt, device=dev), y2=torch.zeros(T, c.width, dtype=f32, device=dev))
+            ws.h2, ws.y2 = b["h2"].data_ptr(), b["y2"].data_ptr()
         if top:
             pairs = T * top
             tiles = (pairs + 15) // 16 + max(ly.experts for ly in c.layers)          # the smallest tile size the forward picks
