@@ -772,18 +772,21 @@ def main():
     ap.add_argument("--phase-timeout", type=float, default=240.0, help="watchdog per pp / tp phase, seconds")
     ap.add_argument("--dry-run", action="store_true", help="launch plumbing only (gloo, no GPU work)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--family", default=None, choices=[None, "gitopel", "fidizen", "tomopel"],
+    ap.add_argument("--family", default=None, choices=[None, "gitopel", "fidizen", "tomopel", "zusuvik"],
                     help="gitopel: prefill / decode throughput of the sequence-mixer family beside Llama at equal size; "
                          "fidizen: of the Fidizen design beside Gitopel's attention layers at equal size; "
-                         "tomopel: of the Tomopel design beside Gitopel at equal size "
+                         "tomopel: of the Tomopel design beside Gitopel at equal size; "
+                         "zusuvik: of the Zusuvik design beside Tomopel at equal size "
                          "(scripts/bench_seqmix.py; one GPU) instead of the headline workload")
     sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "scripts"))
     import bench_seqmix
     bench_seqmix.add_args(ap)
     args = ap.parse_args()
-    if args.family in ("gitopel", "fidizen", "tomopel"):
+    if args.family in ("gitopel", "fidizen", "tomopel", "zusuvik"):
         if args.prompt_len == 128:
             args.prompt_len = 2048
+        if args.family == "zusuvik":
+            return bench_seqmix.run_zusuvik(args)
         if args.family == "tomopel":
             return bench_seqmix.run_tomopel(args)
         return bench_seqmix.run_fidizen(args) if args.family == "fidizen" else bench_seqmix.run(args)

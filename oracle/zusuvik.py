@@ -77,9 +77,11 @@ def retention(X, pos, m: dict, w: dict, eps: float, state=None):
     heads side by side times silu(W_g h), then W_o.  w: q, k, v, g, o.  Returns (out, state [heads, dim, vdim])."""
     H, D, Dv = int(m["heads"]), int(m["dim"]), int(m["vdim"])
     n = X.shape[0]
-    fr = rotary_frequencies(m["rot"])
-    q = rotary((X @ w["q"].T).view(n, H, D), pos, fr, int(m["rot"]["dims"]), "half")
-    k = rotary((X @ w["k"].T).view(n, H, D), pos, fr, int(m["rot"]["dims"]), "half") * D ** -0.5
+    q, k = (X @ w["q"].T).view(n, H, D), (X @ w["k"].T).view(n, H, D)
+    if m.get("rot") and int(m["rot"]["dims"]) > 0:
+        fr = rotary_frequencies(m["rot"])
+        q, k = (rotary(z, pos, fr, int(m["rot"]["dims"]), "half") for z in (q, k))
+    k = k * D ** -0.5
     v = (X @ w["v"].T).view(n, H, Dv)
     decay = torch.tensor([float(d) for d in m["decay"]], dtype=X.dtype)
     S = torch.zeros(H, D, Dv, dtype=X.dtype) if state is None else state.clone()
@@ -192,13 +194,17 @@ def route_top_logits(z, top: int):
     return order, torch.softmax(torch.gather(z, 1, order), dim=-1)
 
 
-def expert_mixture(X, mlp: dict, w: dict):
+def expert_mixture(X, mlp: dict, w: dict, margins=None):
     """routed experts (weights = softmax over the chosen logits, applied to the experts' outputs) plus, where the
-    configuration has one, a shared expert times sigmoid(W_sg h), one number per token"""
+    configuration has one, a shared expert times sigmoid(W_sg h), one number per token.  margins (a list): gets, per token, how
+    far the last chosen logit stands above the first one not chosen."""
     E, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
     limit = float(mlp["expert"]["limit"])
     z = X @ w["router"].T + w["router.b"]
     sel, wt = route_top_logits(z, top)
+    if margins is not None and top < E:
+        srt = torch.sort(z, dim=-1, descending=True).values
+        margins.extend((srt[:, top - 1] - srt[:, top]).tolist())
     y = torch.zeros(X.shape[0], w["e0.down"].shape[0], dtype=X.dtype)
     for e in range(E):
         for c in range(top):
@@ -230,7 +236,7 @@ def _sub(sd: dict, prefix: str, dtype) -> dict:
     return {k[len(prefix):]: v.to(dtype) for k, v in sd.items() if k.startswith(prefix)}
 
 
-def forward(cfg: dict, sd: dict, tokens, state=None, dtype=F):
+def forward(cfg: dict, sd: dict, tokens, state=None, dtype=F, margins=None):
     """tokens: the next ids of ONE sequence; state: what ``forward`` returned for the stretch before (None: the sequence
     starts).  Returns (logits [n, vocab], residual stream after every layer run [runs, n, width], state)."""
     eps = float(cfg["norm"]["eps"])
@@ -261,7 +267,7 @@ def forward(cfg: dict, sd: dict, tokens, state=None, dtype=F):
         new_runs[r] = ns
         if ly.get("mlp"):
             h2 = one_plus_norm(x, sd[p + "norm2"].to(dtype), eps)
-            y = y + expert_mixture(h2, ly["mlp"], _sub(sd, p + "mlp.", dtype))
+            y = y + expert_mixture(h2, ly["mlp"], _sub(sd, p + "mlp.", dtype), margins)
         x = x + y
         trace.append(x.clone())
     logits = one_plus_norm(x, sd["final.norm"].to(dtype), eps) @ emb.T * float(cfg["logit_scale"])

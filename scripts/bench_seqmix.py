@@ -14,6 +14,12 @@ synthetic ids.
         Tomopel has its parallel mixer, gated-linear-attention layers (the same scan kernel) where it has a minGRU -- at
         equal width, heads x head size, feed-forward width and layer count
 
+    python bench.py --family zusuvik [--sizes 1b,8b] ...
+        Zusuvik (parallel blocks; retention layers; convolved capped attention beside a matrix memory; capped-GLU experts routed
+        on the logits with a gated shared expert) beside Tomopel -- the closest existing model: its parallel mixer (attention
+        beside a state-space layer on the same scans) where Zusuvik has its own, minGRU layers where it has retention, routed
+        experts everywhere -- at equal width, heads x head size, state size, expert width and layer count
+
 or directly: python scripts/bench_seqmix.py.  One JSON line: per size, ms and tokens/s of
   prefill   one prompt of --prompt-len tokens in one step (Llama: its chunked prompt path)
   decode    one token per step behind that prompt, batch 1 (both) and batch --batch (Gitopel; the Llama runtime is batch 1)
@@ -62,6 +68,37 @@ TOM_SIZES = {
 }
 
 
+# Zusuvik: "r" layers are retention (r_heads x r_dim keys, r_vdim values), "p" layers convolved attention (heads x dim over
+# kv_heads, `conv` taps) beside a matrix memory (m_heads x m_dim keys, m_vdim values); every layer has experts (each ff / 4
+# wide, two of eight used) and a shared one
+ZUS_SIZES = {
+    "1b": dict(width=2048, ff=8192, heads=32, kv_heads=8, dim=64, vdim=64, conv=4, m_heads=8, m_dim=128, m_vdim=256, r_heads=8,
+               r_dim=128, r_vdim=256, experts=8, top=2, pattern="rprp", vocab=32000),
+    "8b": dict(width=4096, ff=14336, heads=32, kv_heads=8, dim=128, vdim=128, conv=4, m_heads=16, m_dim=128, m_vdim=256, r_heads=16,
+               r_dim=128, r_vdim=256, experts=8, top=2, pattern="rp", vocab=32000),
+}
+
+
+def zusuvik_config(s):
+    layers = []
+    mlp = {"kind": "moe", "router": {"experts": s["experts"], "top": s["top"]}, "expert": {"ff": s["ff"] // 4, "limit": 7.0},
+           "shared": {"ff": s["ff"] // 4, "limit": 7.0}}
+    for ch in s["pattern"]:
+        if ch == "p":
+            mixer = {"left": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["vdim"], "conv": s["conv"],
+                              "rot": {"base": 500000.0, "dims": s["dim"], "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+                              "scale": s["dim"] ** -0.5, "softcap": 30.0},
+                     "right": {"heads": s["m_heads"], "dim": s["m_dim"], "vdim": s["m_vdim"], "gate_cap": 15.0},
+                     "left_scale": 1.0, "right_scale": 1.0}
+            layers.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
+        else:
+            H = s["r_heads"]
+            mixer = {"heads": H, "dim": s["r_dim"], "vdim": s["r_vdim"], "decay": [1.0 - 2.0 ** (-5 - 5 * h / max(H - 1, 1)) for h in range(H)],
+                     "rot": {"base": 10000.0, "dims": s["r_dim"]}}
+            layers.append({"type": "retention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Zusuvik", "layers": layers, "norm": {"eps": 1e-6}, "vocab": s["vocab"], "width": s["width"], "logit_scale": 1.0}
+
+
 def tomopel_config(s):
     layers = []
     for i, ch in enumerate(s["pattern"]):
@@ -73,7 +110,7 @@ def tomopel_config(s):
             kind = "parallel"
         else:
             mixer, kind = {"width": s["width"]}, "mingru"
-        if i % 2 == 0:
+        if i % 2 == 0 and not s.get("all_moe"):
             mlp = {"kind": "dense", "ff": s["ff"]}
         else:
             mlp = {"kind": "moe", "router": {"experts": s["experts"], "top": s["top"]}, "expert": {"ff": s["ff"] // 4},
@@ -141,14 +178,19 @@ def timed(fn, reps):
     return (time.time() - t0) / reps * 1e3
 
 
-def bench_gitopel(s, args, dtype, fidizen=False, tomopel=False):
+def bench_gitopel(s, args, dtype, fidizen=False, tomopel=False, zusuvik=False):
     from umbrella_amd.models import fidizen as fid
     from umbrella_amd.models import gitopel
     from umbrella_amd.models import tomopel as tom
+    from umbrella_amd.models import zusuvik as zus
     B, P, steps = args.batch, args.prompt_len, args.decode_steps
     kw = dict(batch_size=B + 1, max_length=P + 2 * steps + 8, max_tokens=(B + 1) * (P + 2 * steps + 8), device="cuda:0",
               dtype=dtype, max_step_tokens=max(P, B))
-    if tomopel:
+    if zusuvik:
+        cfg = zus.config_from_dict(zusuvik_config(s))
+        sd = device_state(cfg, dtype, shapes=zus.tensor_shapes(cfg), zero_norms=True)
+        m = zus.Zusuvik("bench", state_dict=sd, config=cfg, **kw)
+    elif tomopel:
         cfg = tom.config_from_dict(tomopel_config(s))
         sd = device_state(cfg, dtype, shapes=tom.tensor_shapes(cfg, s["bias_rows"]), zero_norms=True)
         m = tom.Tomopel("bench", state_dict=sd, config=cfg, **kw)
@@ -263,6 +305,31 @@ def run_tomopel(args):
     return line
 
 
+def run_zusuvik(args):
+    """Zusuvik beside Tomopel at equal width, heads x head size, state size, expert width and layer count: Tomopel's parallel
+    mixer for Zusuvik's, minGRU layers for the retention layers, routed experts in every layer"""
+    import __graft_entry__ as ge
+    ge.build_seq()
+    dtype = torch.bfloat16
+    res = {}
+    for name in args.sizes.split(","):
+        s = ZUS_SIZES[name]
+        res[name] = {"shape": dict(s)}
+        res[name]["zusuvik"] = bench_gitopel(s, args, dtype, zusuvik=True)
+        torch.cuda.empty_cache()
+        if not args.no_gitopel:
+            t = dict(width=s["width"], ff=s["ff"], heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["vdim"],
+                     s_heads=s["m_heads"] * 4, s_vdim=s["m_vdim"] // 4, state=s["m_dim"], groups=8, conv=s["conv"], experts=s["experts"],
+                     top=s["top"], pattern=s["pattern"].replace("r", "g"), vocab=s["vocab"], bias_rows=32, bias_max=2048, all_moe=True)
+            res[name]["tomopel_equal_size"] = bench_gitopel(t, args, dtype, tomopel=True)
+            torch.cuda.empty_cache()
+    line = {"metric": "prefill / decode throughput, Zusuvik beside Tomopel at equal size", "unit": "tokens/s",
+            "dtype": "bf16", "data": "synthetic: random weights, random ids", "n_gpus": 1, "prompt_len": args.prompt_len,
+            "decode_steps": args.decode_steps, "batch": args.batch, "sizes": res}
+    print(json.dumps(line), flush=True)
+    return line
+
+
 def run(args):
     import __graft_entry__ as ge
     ge.build()
@@ -295,7 +362,7 @@ def add_args(ap):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--prompt-len", type=int, default=2048)
-    ap.add_argument("--family", default="gitopel", choices=["gitopel", "fidizen", "tomopel"])
+    ap.add_argument("--family", default="gitopel", choices=["gitopel", "fidizen", "tomopel", "zusuvik"])
     add_args(ap)
     a = ap.parse_args()
-    {"fidizen": run_fidizen, "tomopel": run_tomopel}.get(a.family, run)(a)
+    {"fidizen": run_fidizen, "tomopel": run_tomopel, "zusuvik": run_zusuvik}.get(a.family, run)(a)

@@ -153,6 +153,8 @@ def test_seq_header_matches_the_bindings():
     assert C.sizeof(_lib.UmbSeqLinear) == 24 and C.sizeof(_lib.UmbPagedKV) == 56
     base = 16 * 4 + 5 * 24 + 7 * 8 + 56 + 8 + 8 * 4 + 24 + 10 * 8 + 24 + 2 * 8 + 2 * 24
     # + activation / routing kinds and correction, stream tables, the distance-bias attention and state-space fields
-    assert C.sizeof(_lib.UmbSeqLayer) == base + (2 * 4 + 8) + 6 * 8 + (3 * 8 + 2 * 4 + 4 * 4) + (6 * 4 + 7 * 8)
-    assert C.sizeof(_lib.UmbSeqModel) == 32 + 16 + 24 + 8 + 16 and C.sizeof(_lib.UmbSeqWork) == 9 * 8 + 8 + 8 * 8 + 8
+    # + the retention / convolved-attention / matrix-memory fields, the capped activation's constants, the embedding flag
+    assert C.sizeof(_lib.UmbSeqLayer) == base + (2 * 4 + 8) + 6 * 8 + (3 * 8 + 2 * 4 + 4 * 4) + (6 * 4 + 7 * 8) + \
+        (8 + 4 * 4 + 2 * 8 + 4 * 4 + 2 * 8 + 4 * 4 + 2 * 4)
+    assert C.sizeof(_lib.UmbSeqModel) == 32 + 16 + 24 + 8 + 16 + 8 and C.sizeof(_lib.UmbSeqWork) == 9 * 8 + 8 + 8 * 8 + 8 + 2 * 8
     assert C.sizeof(_lib.UmbSeqStep) == 16 + 9 * 8

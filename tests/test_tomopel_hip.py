@@ -322,13 +322,13 @@ def _run_attn(lib, X, w, dtype, splits, H, G, D, E, scale, far, temp, eps, page=
         nd = bias.shape[1] if bias is not None else 0
         if cnt >= 16 and lib.umb_bsa_attend_tiled_ok(H, G, D, E, code(dtype)):       # as the forward chooses: the matrix pipe
             _lib.seq_call("umb_bsa_attend_tiled", out, H * E + 3, q, kv, proj, ld, H * D + G * D + G * E, bias, nd, st.d["seq_slot"],
-                          st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, cnt, H, G, D, E, window, scale, out_scale, code(dtype))
+                          st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, cnt, H, G, D, E, window, scale, out_scale, 0.0, code(dtype))
         else:
             # steps of few rows with scratch: the keys of a row are dealt to several workgroups and merged
             need = cnt * H * 16 * (E + 2) if split_keys else 0
             scratch = torch.zeros(max(need, 1), dtype=torch.float32, device="cuda:0") if split_keys else None
             _lib.seq_call("umb_bsa_attend", out, H * E + 3, q, kv, proj, ld, H * D + G * D + G * E, bias, nd, st.d["pos"],
-                          st.d["slot"], cnt, H, G, D, E, window, scale, out_scale, scratch, need, code(dtype))
+                          st.d["slot"], cnt, H, G, D, E, window, scale, out_scale, 0.0, scratch, need, code(dtype))
         assert float(out[:, H * E:].abs().max()) == 0.0
         outs.append(out[:, :H * E].clone())
         at += cnt

@@ -48,8 +48,8 @@ def _mixer(kind: str, m: dict):
         a, b = m["left"], m["right"]
         dims, base, scaling = _rot(a)
         return AttnMLSTMCfg(heads=int(a["heads"]), kv_heads=int(a.get("kv_heads", a["heads"])), dim=int(a["dim"]),
-                            vdim=int(a.get("vdim", a["dim"])), scale=float(a["scale"]), softcap=float(a.get("softcap", 0.0)),
-                            taps=int(a.get("conv", 1)), rot_dims=dims, rot_base=base, rot_scaling=scaling,
+                            vdim=int(a.get("vdim", a["dim"])), scale=float(a["scale"]), softcap=float(a.get("softcap") or 0.0),
+                            window=int(a.get("window") or 0), taps=int(a.get("conv") or 1), rot_dims=dims, rot_base=base, rot_scaling=scaling,
                             rot_layout="interleaved", a_scale=float(m.get("left_scale", 1.0)), m_heads=int(b["heads"]),
                             m_dim=int(b["dim"]), m_vdim=int(b.get("vdim", b["dim"])), gate_cap=float(b["gate_cap"]),
                             b_scale=float(m.get("right_scale", 1.0)))
