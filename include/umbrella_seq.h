@@ -326,17 +326,17 @@ int umb_cva_prep(float* q, const UmbPagedKV* kv, const float* proj, int ld, cons
                  const void* w_k, const int* pos, const int* slot, const float* freq, int T, int H, int G, int D, int E, int taps,
                  int rot_dims, int layout, int update_state, float eps, int dtype, umb_stream_t stream);
 
-/* ---- matrix memory with exponential gates.  gates fp32 [T][2 H] = [i | f]: i = cap tanh(z_i / cap), f = log sigmoid(cap
- * tanh(z_f / cap)) from columns i_col / f_col of proj.  mscan: m_t = max(f_t + m_(t-1), i_t) token by token per (sequence, head)
- * (mstate fp32 [slots][H]; a sequence that starts at position 0 starts from m = 0); log_alpha[t][h] = f_t + m_(t-1) - m_t, alpha
- * its exponential, mrun[t][h] = m_t.  prep: qs fp32 [T][H D] = q * qscale; vp fp32 [T][H][Pp] = [e^(i - m) v | e^(i - m) | 0 ..]
- * (Pp > Dv): a linear scan over (qs, k, vp, alpha) carries the matrix state and, as value column Dv, the normaliser.
- * step: all three for steps of one token per sequence. */
-int umb_mlstm_gates(float* gates, const float* proj, int ld, int i_col, int f_col, int T, int H, float cap, umb_stream_t stream);
-int umb_mlstm_mscan(float* log_alpha, float* alpha, float* mrun, float* mstate, const float* gates, const int* seq_slot,
-                    const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int H, umb_stream_t stream);
-int umb_mlstm_prep(float* qs, float* vp, const float* proj, int ld, int q_col, int v_col, const float* gates, const float* mrun,
-                   int T, int H, int D, int Dv, int Pp, float qscale, umb_stream_t stream);
+/* ---- matrix memory with exponential gates.  Per (token, head), from columns i_col / f_col of proj: i = cap tanh(z_i / cap),
+ * f = log sigmoid(cap tanh(z_f / cap)).  mscan: the running maximum m_t = max(f_t + m_(t-1), i_t) of every stretch (tiles of 64 tokens
+ * scanned side by side; mstate fp32 [slots][H]; a sequence that starts at position 0 starts from m = 0); log_alpha[t][h] =
+ * f_t + m_(t-1) - m_t, alpha its exponential, mrun[t][h] = m_t, bw[t][h] = e^(i_t - m_t).  prep: qs fp32 [T][H D] = q * qscale;
+ * vp fp32 [T][H][Pp] = [bw v | bw | 0 ..] (Pp > Dv): a linear scan over (qs, k, vp, alpha) carries the matrix state and, as value
+ * column Dv, the normaliser.  step: both for steps of one token per sequence. */
+int umb_mlstm_mscan(float* log_alpha, float* alpha, float* mrun, float* bw, float* mstate, const float* proj, int ld, int i_col,
+                    int f_col, float cap, const int* seq_slot, const int* seq_row0, const int* seq_pos0, const int* seq_len, int B,
+                    int H, umb_stream_t stream);
+int umb_mlstm_prep(float* qs, float* vp, const float* proj, int ld, int q_col, int v_col, const float* bw, int T, int H, int D,
+                   int Dv, int Pp, float qscale, umb_stream_t stream);
 int umb_mlstm_step(float* qs, float* vp, float* log_alpha, float* alpha, float* mrun, float* mstate, const float* proj, int ld,
                    int q_col, int v_col, int i_col, int f_col, const int* pos, const int* slot, int T, int H, int D, int Dv, int Pp,
                    float qscale, float cap, umb_stream_t stream);

@@ -347,16 +347,16 @@ def _run_memory(lib, m, w, X, splits, dtype, slot=2, state=None):
     for cnt in splits:
         st = Steps([cnt], [at], [slot])
         proj = dev(proj_all[at:at + cnt])
-        qs, vp, gates = zeros(cnt, H * D), zeros(cnt, H * Pp), zeros(cnt, 2 * H)
+        qs, vp, bw = zeros(cnt, H * D), zeros(cnt, H * Pp), zeros(cnt, H)
         alpha, la, mrun = zeros(cnt, H), zeros(cnt, H), zeros(cnt, H)
         o, out = zeros(cnt, H * Pp), zeros(cnt, H * Dv + 2, dtype=dtype)
         if cnt == 1:
             call("umb_mlstm_step", qs, vp, la, alpha, mrun, mx, proj, ld, qc, vc, ic, fc, st.d["pos"], st.d["slot"], cnt, H, D, Dv, Pp,
                  D ** -0.5, cap)
         else:
-            call("umb_mlstm_gates", gates, proj, ld, ic, fc, cnt, H, cap)
-            call("umb_mlstm_mscan", la, alpha, mrun, mx, gates, st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"], st.d["seq_len"], 1, H)
-            call("umb_mlstm_prep", qs, vp, proj, ld, qc, vc, gates, mrun, cnt, H, D, Dv, Pp, D ** -0.5)
+            call("umb_mlstm_mscan", la, alpha, mrun, bw, mx, proj, ld, ic, fc, cap, st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"],
+                 st.d["seq_len"], 1, H)
+            call("umb_mlstm_prep", qs, vp, proj, ld, qc, vc, bw, cnt, H, D, Dv, Pp, D ** -0.5)
         _scan(lib, o, S, qs, H * D, _offset(proj, kc), ld, vp, H * Pp, alpha, la, st, H, D, Pp, scratch)
         call("umb_head_gate", out, H * Dv + 2, o, Pp, Dv, mrun, proj, ld, gc, dev(w["norm"], dtype), 1, 1, cnt, H, Dv, 1e-5, 1.2, code(dtype))
         assert float(out[:, H * Dv:].abs().max()) == 0.0

@@ -10,33 +10,70 @@
 // One workgroup per token; the convolved q | k row lives in LDS between the sum of squares and the rotation.  All fp32.
 #include "seq_common.h"
 
-template <typename P>
-__global__ __launch_bounds__(256) void cva_prep_kernel(float* __restrict__ q, UmbPagedKV kv, const float* __restrict__ proj, int ld,
-                                                       const typename El<P>::type* __restrict__ conv_w, float* __restrict__ conv_state,
-                                                       const typename El<P>::type* __restrict__ w_q,
-                                                       const typename El<P>::type* __restrict__ w_k, const int* __restrict__ pos,
-                                                       const int* __restrict__ slot_, const float* __restrict__ freq, int H, int G,
-                                                       int D, int E, int taps, int rot_dims, int layout, int update, float eps) {
+constexpr int CVA_MAXT = 8;      // taps whose loads are issued together (more: a plain loop)
+
+// NT threads per token: 256 when the step has many tokens, 1024 when it has few (a decoding step is a handful of workgroups
+// that each walk thousands of channels).  The taps of a channel are loaded unconditionally from clamped addresses -- the
+// same step's rows or the ring -- before any is used: a load that sits behind a per-tap branch waits for its own round trip.
+template <typename P, int NT>
+__global__ __launch_bounds__(NT) void cva_prep_kernel(float* __restrict__ q, UmbPagedKV kv, const float* __restrict__ proj, int ld,
+                                                      const typename El<P>::type* __restrict__ conv_w, float* __restrict__ conv_state,
+                                                      const typename El<P>::type* __restrict__ w_q,
+                                                      const typename El<P>::type* __restrict__ w_k, const int* __restrict__ pos,
+                                                      const int* __restrict__ slot_, const float* __restrict__ freq, int H, int G,
+                                                      int D, int E, int taps, int rot_dims, int layout, int update, float eps) {
   typedef typename El<P>::type El_;
   extern __shared__ float row_s[];                      // [H D + G D]
-  __shared__ float red[8];
+  __shared__ float red[NT / 64];
   const int t = blockIdx.x, p = pos[t], slot = slot_[t];
   const int nq = H * D, nk = G * D, C = nq + nk + G * E;
+  // where tap j (looking d = taps - 1 - j positions back) comes from: bit j of `same`: a row of this step; of `live`: not
+  // before the sequence's start
+  unsigned same = 0, live = 0;
+  if (conv_w && taps <= CVA_MAXT) {
+    for (int j = 0; j < taps; ++j) {
+      const int d = taps - 1 - j;
+      if (d <= p) {
+        live |= 1u << j;
+        if (d == 0 || (t - d >= 0 && slot_[t - d] == slot)) same |= 1u << j;
+      }
+    }
+  }
+  const long ring0 = (long)slot * (taps - 1);
   float ssq = 0.f, ssk = 0.f;
-  for (int c = threadIdx.x; c < C; c += 256) {
+  // nothing is stored to global fp32 memory inside this loop (the ring is refreshed after it), so the loads of several
+  // channels overlap
+#pragma unroll 4
+  for (int c = threadIdx.x; c < C; c += NT) {
     float acc;
-    if (conv_w) {
+    if (conv_w && taps <= CVA_MAXT) {
+      float in[CVA_MAXT], wv[CVA_MAXT];
+#pragma unroll
+      for (int j = 0; j < CVA_MAXT; ++j) {
+        if (j < taps) {
+          const int d = taps - 1 - j;
+          const bool sm = (same >> j) & 1u, lv = (live >> j) & 1u;
+          const float* src = (sm || !lv) ? proj + (long)(t - (sm ? d : 0)) * ld + c
+                                         : conv_state + (ring0 + (p - d) % (taps - 1)) * C + c;
+          in[j] = *src;
+          wv[j] = ldf<P>(conv_w + (long)c * taps + j);
+        }
+      }
+      acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < CVA_MAXT; ++j)
+        if (j < taps) acc += wv[j] * (((live >> j) & 1u) ? in[j] : 0.f);      // oldest tap first
+    } else if (conv_w) {
       acc = 0.f;
       for (int j = 0; j < taps; ++j) {
         const int d = taps - 1 - j;                       // how far back the tap looks
         float in = 0.f;
         if (d <= p) {
           if (d == 0 || (t - d >= 0 && slot_[t - d] == slot)) in = proj[(long)(t - d) * ld + c];        // same step
-          else in = conv_state[((long)slot * (taps - 1) + (p - d) % (taps - 1)) * C + c];
+          else in = conv_state[(ring0 + (p - d) % (taps - 1)) * C + c];
         }
         acc += ldf<P>(conv_w + (long)c * taps + j) * in;
       }
-      if (update && taps > 1) conv_state[((long)slot * (taps - 1) + p % (taps - 1)) * C + c] = proj[(long)t * ld + c];
     } else {
       acc = proj[(long)t * ld + c];
     }
@@ -47,11 +84,14 @@ __global__ __launch_bounds__(256) void cva_prep_kernel(float* __restrict__ q, Um
       stf<P>(reinterpret_cast<El_*>(kv.v) + pkv_tok(kv, slot, p, g, G, E) + e, acc);
     }
   }
-  ssq = block_sum<256>(ssq, red);
-  ssk = block_sum<256>(ssk, red);                        // its first barrier comes after every read of the first sum
+  // steps of one token per sequence: the ring row of this position held the oldest tap, which the same thread has read above
+  if (update && conv_w && taps > 1)
+    for (int c = threadIdx.x; c < C; c += NT) conv_state[(ring0 + p % (taps - 1)) * C + c] = proj[(long)t * ld + c];
+  ssq = block_sum<NT>(ssq, red);
+  ssk = block_sum<NT>(ssk, red);                         // its first barrier comes after every read of the first sum
   const float fq = 1.f / sqrtf(ssq / (float)nq + eps), fk = 1.f / sqrtf(ssk / (float)nk + eps);
   const int half = rot_dims >> 1;
-  for (int c = threadIdx.x; c < nq + nk; c += 256) {
+  for (int c = threadIdx.x; c < nq + nk; c += NT) {
     const bool is_q = c < nq;
     const int cc = is_q ? c : c - nq;
     const int h = cc / D, d = cc - h * D;
@@ -86,9 +126,15 @@ extern "C" int umb_cva_prep(float* q, const UmbPagedKV* kv, const float* proj, i
   if (lds > 160 * 1024 - 64) return UMB_EINVAL;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type El_;
-    if (ensure_dynamic_lds<cva_prep_kernel<P>>(lds) != UMB_OK) return UMB_EHIP;
-    hipLaunchKernelGGL(cva_prep_kernel<P>, dim3(T), dim3(256), lds, st, q, *kv, proj, ld, (const El_*)conv_w, conv_state,
-                       (const El_*)w_q, (const El_*)w_k, pos, slot, freq, H, G, D, E, taps, rot_dims, layout, update_state, eps);
+    if (T <= 64) {
+      if (ensure_dynamic_lds<cva_prep_kernel<P, 1024>>(lds) != UMB_OK) return UMB_EHIP;
+      hipLaunchKernelGGL((cva_prep_kernel<P, 1024>), dim3(T), dim3(1024), lds, st, q, *kv, proj, ld, (const El_*)conv_w, conv_state,
+                         (const El_*)w_q, (const El_*)w_k, pos, slot, freq, H, G, D, E, taps, rot_dims, layout, update_state, eps);
+    } else {
+      if (ensure_dynamic_lds<cva_prep_kernel<P, 256>>(lds) != UMB_OK) return UMB_EHIP;
+      hipLaunchKernelGGL((cva_prep_kernel<P, 256>), dim3(T), dim3(256), lds, st, q, *kv, proj, ld, (const El_*)conv_w, conv_state,
+                         (const El_*)w_q, (const El_*)w_k, pos, slot, freq, H, G, D, E, taps, rot_dims, layout, update_state, eps);
+    }
   })
   UMB_LAUNCH_CHECK();
   return UMB_OK;

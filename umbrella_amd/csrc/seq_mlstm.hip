@@ -6,70 +6,70 @@
 // linear recurrence S <- a S + k (b v)^T with one decay per head, and n is the same recurrence with the value 1: the normaliser
 // rides along as ONE EXTRA VALUE COLUMN (v' = [b v | b | 0 ..], Pp columns), so the scans of seq_gla.hip / seq_ssd.hip carry both
 // and the read-out's column Dv is n . q.  This file holds what is special:
-//   gates   i and f of every (token, head), side by side
-//   mscan   the running maximum, token by token per (sequence, head) -- two dependent operations a token, in the order the
-//           equations give, so its bits never depend on how a prompt was cut; leaves log a, a and m for every token and the last m
-//           in the sequence's slot (a sequence that starts at position 0 starts from m = 0 whatever its slot holds)
+//   mscan   the gates and the running maximum of every (token, head): leaves log a, a, m and b for every token and the last m in
+//           the sequence's slot (a sequence that starts at position 0 starts from m = 0 whatever its slot holds)
 //   prep    scaled queries and the widened value rows
-//   step    all three for steps of one token per sequence, in one launch
+//   step    both for steps of one token per sequence, in one launch
 // The stabilised division, the per-head norm and the output gate are head_gate of seq_retention.hip.  Everything is fp32.
 #include "seq_common.h"
 
 __device__ __forceinline__ float mlstm_gate_i(float z, float cap) { return cap * tanhf(z / cap); }
 __device__ __forceinline__ float mlstm_gate_f(float z, float cap) { return log_sigmoidf_(cap * tanhf(z / cap)); }
 
-__global__ __launch_bounds__(256) void mlstm_gates_kernel(float* __restrict__ gates, const float* __restrict__ proj, int ld, int i_col,
-                                                          int f_col, long n, int H, float cap) {
-  const long x = (long)blockIdx.x * 256 + threadIdx.x;
-  if (x >= n) return;
-  const long t = x / H;
-  const int h = (int)(x - t * H);
-  gates[t * 2 * H + h] = mlstm_gate_i(proj[t * ld + i_col + h], cap);
-  gates[t * 2 * H + H + h] = mlstm_gate_f(proj[t * ld + f_col + h], cap);
-}
-
+// One wave per (sequence, head) walks the stretch in tiles of 64 tokens, lane = token.  The recurrence m <- max(f + m, i) is the
+// composition of the maps m -> max(m + a, b); two of them compose to (a1 + a2, max(b1 + a2, b2)), so a tile is an inclusive scan
+// over the lanes (six exchanges) applied to the maximum the tile inherits.  The gates are formed here (lane = token: tanh and
+// log-sigmoid side by side), the next tile's projections are in flight while the current one is scanned.  Against the
+// token-by-token order the sums f + f + .. are associated differently: the maxima agree to fp32 rounding, and since every
+// decay and weight below is formed from the SAME maxima the recurrence they describe is the same.
 __global__ __launch_bounds__(64) void mlstm_mscan_kernel(float* __restrict__ log_alpha, float* __restrict__ alpha,
-                                                         float* __restrict__ mrun, float* __restrict__ mstate,
-                                                         const float* __restrict__ gates, const int* __restrict__ seq_slot,
+                                                         float* __restrict__ mrun, float* __restrict__ bw,
+                                                         float* __restrict__ mstate, const float* __restrict__ proj, int ld, int i_col,
+                                                         int f_col, float cap, const int* __restrict__ seq_slot,
                                                          const int* __restrict__ seq_row0, const int* __restrict__ seq_pos0,
-                                                         const int* __restrict__ seq_len, int B, int H) {
-  const int x = blockIdx.x * 64 + threadIdx.x;
-  if (x >= B * H) return;
-  const int b = x / H, h = x - b * H;
+                                                         const int* __restrict__ seq_len, int H) {
+  const int b = blockIdx.x / H, h = blockIdx.x - b * H, lane = threadIdx.x;
   const int n = seq_len[b];
   if (n <= 0) return;
   const long row0 = seq_row0[b];
   float* ms = mstate + (long)seq_slot[b] * H + h;
-  float m = seq_pos0[b] == 0 ? 0.f : *ms;
-  constexpr int U = 8;                                   // gates of eight tokens in flight ahead of the dependent chain
-  for (int t0 = 0; t0 < n; t0 += U) {
-    float gi[U], gf[U];
+  float m_in = seq_pos0[b] == 0 ? 0.f : *ms;
+  auto fetch = [&](int t0, float& zi, float& zf) {
+    const long r = row0 + (t0 + lane < n ? t0 + lane : n - 1);        // clamped: never used past the stretch
+    zi = proj[r * ld + i_col + h];
+    zf = proj[r * ld + f_col + h];
+  };
+  float zi, zf;
+  fetch(0, zi, zf);
+  for (int t0 = 0; t0 < n; t0 += 64) {
+    const float gi = mlstm_gate_i(zi, cap), gf = mlstm_gate_f(zf, cap);
+    if (t0 + 64 < n) fetch(t0 + 64, zi, zf);
+    const bool live = t0 + lane < n;
+    float a = live ? gf : 0.f, bb = live ? gi : -INFINITY;           // past the stretch: the identity map
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const long r = row0 + (t0 + u < n ? t0 + u : n - 1);
-      gi[u] = gates[r * 2 * H + h];
-      gf[u] = gates[r * 2 * H + H + h];
+    for (int o = 1; o < 64; o <<= 1) {
+      const float pa = __shfl_up(a, o, 64), pb = __shfl_up(bb, o, 64);
+      if (lane >= o) { bb = fmaxf(pb + a, bb); a = pa + a; }
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (t0 + u < n) {
-        const float carried = gf[u] + m;
-        const float mn = fmaxf(carried, gi[u]);
-        const float la = carried - mn;
-        const long r = row0 + t0 + u;
-        log_alpha[r * H + h] = la;
-        alpha[r * H + h] = expf(la);
-        mrun[r * H + h] = mn;
-        m = mn;
-      }
+    const float m = fmaxf(a + m_in, bb);
+    float mp = __shfl_up(m, 1, 64);
+    if (lane == 0) mp = m_in;
+    if (live) {
+      const long r = row0 + t0 + lane;
+      const float la = gf + mp - m;
+      log_alpha[r * H + h] = la;
+      alpha[r * H + h] = expf(la);
+      mrun[r * H + h] = m;
+      bw[r * H + h] = expf(gi - m);
     }
+    m_in = __shfl(m, 63, 64);                                        // past the stretch the map is the identity: lane 63 holds the last m
   }
-  *ms = m;
+  if (lane == 0) *ms = m_in;
 }
 
 __global__ __launch_bounds__(256) void mlstm_prep_kernel(float* __restrict__ qs, float* __restrict__ vp, const float* __restrict__ proj,
-                                                         int ld, int q_col, int v_col, const float* __restrict__ gates,
-                                                         const float* __restrict__ mrun, int H, int D, int Dv, int Pp, float qscale) {
+                                                         int ld, int q_col, int v_col, const float* __restrict__ bw, int H, int D,
+                                                         int Dv, int Pp, float qscale) {
   const int t = blockIdx.x, idx = blockIdx.y * 256 + threadIdx.x;
   const int nq = H * D;
   if (idx < nq) {
@@ -79,8 +79,8 @@ __global__ __launch_bounds__(256) void mlstm_prep_kernel(float* __restrict__ qs,
   const int j = idx - nq;
   if (j >= H * Pp) return;
   const int h = j / Pp, c = j - h * Pp;
-  const float bw = expf(gates[(long)t * 2 * H + h] - mrun[(long)t * H + h]);
-  vp[(long)t * H * Pp + j] = c < Dv ? bw * proj[(long)t * ld + v_col + (long)h * Dv + c] : (c == Dv ? bw : 0.f);
+  const float w = bw[(long)t * H + h];
+  vp[(long)t * H * Pp + j] = c < Dv ? w * proj[(long)t * ld + v_col + (long)h * Dv + c] : (c == Dv ? w : 0.f);
 }
 
 // one token per sequence: gates, maximum, decays, scaled query and widened value row of a (token, head) by one workgroup slice
@@ -110,32 +110,25 @@ __global__ __launch_bounds__(256) void mlstm_step_kernel(float* __restrict__ qs,
     vp[(long)t * H * Pp + (long)h * Pp + c] = c < Dv ? bw * proj[(long)t * ld + v_col + (long)h * Dv + c] : (c == Dv ? bw : 0.f);
 }
 
-extern "C" int umb_mlstm_gates(float* gates, const float* proj, int ld, int i_col, int f_col, int T, int H, float cap,
-                               hipStream_t st) {
-  if (T < 1 || H < 1 || !(cap > 0.f) || !gates || !proj || i_col < 0 || f_col < 0 || ld < i_col + H || ld < f_col + H) return UMB_EINVAL;
-  const long n = (long)T * H;
-  hipLaunchKernelGGL(mlstm_gates_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gates, proj, ld, i_col, f_col, n, H, cap);
-  UMB_LAUNCH_CHECK();
-  return UMB_OK;
-}
-
-extern "C" int umb_mlstm_mscan(float* log_alpha, float* alpha, float* mrun, float* mstate, const float* gates, const int* seq_slot,
-                               const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int H, hipStream_t st) {
-  if (B < 1 || H < 1 || !log_alpha || !alpha || !mrun || !mstate || !gates || !seq_slot || !seq_row0 || !seq_pos0 || !seq_len)
+extern "C" int umb_mlstm_mscan(float* log_alpha, float* alpha, float* mrun, float* bw, float* mstate, const float* proj, int ld,
+                               int i_col, int f_col, float cap, const int* seq_slot, const int* seq_row0, const int* seq_pos0,
+                               const int* seq_len, int B, int H, hipStream_t st) {
+  if (B < 1 || H < 1 || !(cap > 0.f) || !log_alpha || !alpha || !mrun || !bw || !mstate || !proj || !seq_slot || !seq_row0 ||
+      !seq_pos0 || !seq_len || i_col < 0 || f_col < 0 || ld < i_col + H || ld < f_col + H)
     return UMB_EINVAL;
-  hipLaunchKernelGGL(mlstm_mscan_kernel, dim3((B * H + 63) / 64), dim3(64), 0, st, log_alpha, alpha, mrun, mstate, gates, seq_slot,
-                     seq_row0, seq_pos0, seq_len, B, H);
+  hipLaunchKernelGGL(mlstm_mscan_kernel, dim3(B * H), dim3(64), 0, st, log_alpha, alpha, mrun, bw, mstate, proj, ld, i_col, f_col, cap,
+                     seq_slot, seq_row0, seq_pos0, seq_len, H);
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }
 
-extern "C" int umb_mlstm_prep(float* qs, float* vp, const float* proj, int ld, int q_col, int v_col, const float* gates,
-                              const float* mrun, int T, int H, int D, int Dv, int Pp, float qscale, hipStream_t st) {
-  if (T < 1 || H < 1 || D < 1 || Dv < 1 || Pp < Dv + 1 || !qs || !vp || !proj || !gates || !mrun || q_col < 0 || v_col < 0 ||
+extern "C" int umb_mlstm_prep(float* qs, float* vp, const float* proj, int ld, int q_col, int v_col, const float* bw, int T, int H,
+                              int D, int Dv, int Pp, float qscale, hipStream_t st) {
+  if (T < 1 || H < 1 || D < 1 || Dv < 1 || Pp < Dv + 1 || !qs || !vp || !proj || !bw || q_col < 0 || v_col < 0 ||
       ld < q_col + H * D || ld < v_col + H * Dv)
     return UMB_EINVAL;
-  hipLaunchKernelGGL(mlstm_prep_kernel, dim3(T, (H * (D + Pp) + 255) / 256), dim3(256), 0, st, qs, vp, proj, ld, q_col, v_col, gates,
-                     mrun, H, D, Dv, Pp, qscale);
+  hipLaunchKernelGGL(mlstm_prep_kernel, dim3(T, (H * (D + Pp) + 255) / 256), dim3(256), 0, st, qs, vp, proj, ld, q_col, v_col, bw, H, D,
+                     Dv, Pp, qscale);
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }

@@ -11,7 +11,7 @@
 //                norms + temperature + append | attend  ||  convolution + dt + decay | state ring | scan | gate + norm
 //     retention: proj GEMM ([q | k | v | g]) | rotary + constants | decay rows | scan | per-head unit RMS * SiLU gate | out GEMM
 //     convolved attention beside a matrix memory (one fused proj GEMM, one out GEMM over [a | b]):
-//                convolution + whole-row norms + rotary + append | ring | attend (capped scores)  ||  gates | running maximum |
+//                convolution + whole-row norms + rotary + append | ring | attend (capped scores)  ||  gates + running maximum |
 //                scaled queries + widened values | scan | stabilised division + per-head norm + sigmoid gate
 // Stacks whose two sublayers read the SAME residual (UmbSeqModel.block = UMB_BLOCK_PARALLEL) run mixer and feed-forward from two
 // normed inputs and meet in one seam per layer; a layer may ask for the embedding row to be added again in front of it.
@@ -225,11 +225,11 @@ static int mix_attn_mlstm(const UmbSeqModel* m, const UmbSeqLayer& ly, const Umb
   const int mq = C, mk = mq + Hm * Dm, mv = mk + Hm * Dm, mg = mv + Hm * Em, ic = mg + Hm * Em, fc = ic + Hm;
   const int ldo = H * E + Hm * Em;
   if (ld != fc + Hm || ly.out.K != ldo || !ly.state || !ly.m_max || ly.c_taps < 1) return UMB_EINVAL;
-  float* q = ws->aux;                                        // [T][H D] | qs | vp | gates | alpha | log alpha | m | scratch
+  float* q = ws->aux;                                        // [T][H D] | qs | vp | input weights | alpha | log alpha | m | scratch
   float* qs = q + al4((long)T * H * D);
   float* vp = qs + al4((long)T * Hm * Dm);
-  float* gates = vp + al4((long)T * Hm * Pp);
-  float* alpha = gates + al4((long)T * 2 * Hm);
+  float* bw = vp + al4((long)T * Hm * Pp);
+  float* alpha = bw + al4((long)T * Hm);
   float* log_alpha = alpha + al4((long)T * Hm);
   float* mrun = log_alpha + al4((long)T * Hm);
   float* spare2 = mrun + al4((long)T * Hm);
@@ -251,9 +251,9 @@ static int mix_attn_mlstm(const UmbSeqModel* m, const UmbSeqLayer& ly, const Umb
     SEQ_TRY(umb_mlstm_step(qs, vp, log_alpha, alpha, mrun, ly.m_max, ws->proj, ld, mq, mv, ic, fc, s->pos, s->slot, T, Hm, Dm, Em, Pp,
                            qscale, ly.gate_cap, st));
   else {
-    SEQ_TRY(umb_mlstm_gates(gates, ws->proj, ld, ic, fc, T, Hm, ly.gate_cap, st));
-    SEQ_TRY(umb_mlstm_mscan(log_alpha, alpha, mrun, ly.m_max, gates, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B, Hm, st));
-    SEQ_TRY(umb_mlstm_prep(qs, vp, ws->proj, ld, mq, mv, gates, mrun, T, Hm, Dm, Em, Pp, qscale, st));
+    SEQ_TRY(umb_mlstm_mscan(log_alpha, alpha, mrun, bw, ly.m_max, ws->proj, ld, ic, fc, ly.gate_cap, s->seq_slot, s->seq_row0, s->seq_pos0,
+                            s->seq_len, s->B, Hm, st));
+    SEQ_TRY(umb_mlstm_prep(qs, vp, ws->proj, ld, mq, mv, bw, T, Hm, Dm, Em, Pp, qscale, st));
   }
   SEQ_TRY(scan_per_head(ws->o, ly.state, qs, Hm * Dm, ws->proj + mk, ld, vp, Hm * Pp, alpha, log_alpha, s, Hm, Dm, Pp, spare2,
                         spare2_floats, st));
