@@ -321,10 +321,13 @@ int umb_head_gate(void* out, int ldo, const float* o, int P_cols, int den_col, c
  * steps' inputs from conv_state fp32 [slots][taps - 1][C], position p in row p % (taps - 1)); q and k are RMS-normed over their
  * WHOLE rows (weights w_q [H D], w_k [G D], null: 1) and rotated (rot_dims, layout and freq as umb_rope_scale); q -> fp32
  * [T][H D], k and v -> the paged store.  The ring is refreshed by umb_ssd_conv_update (col0 0) afterwards, or here with
- * update_state (steps of ONE token per sequence only).  The attention is umb_bsa_attend with a softcap. */
+ * update_state (steps of ONE token per sequence only).  scratch (fp32, may be null): with T (H D + G D + 2 ceil(C / 256)) floats
+ * of it, steps of at most 64 tokens run as two launches over (token, 256 channels) instead of one workgroup per token.  The
+ * attention is umb_bsa_attend with a softcap. */
 int umb_cva_prep(float* q, const UmbPagedKV* kv, const float* proj, int ld, const void* conv_w, float* conv_state, const void* w_q,
                  const void* w_k, const int* pos, const int* slot, const float* freq, int T, int H, int G, int D, int E, int taps,
-                 int rot_dims, int layout, int update_state, float eps, int dtype, umb_stream_t stream);
+                 int rot_dims, int layout, int update_state, float eps, float* scratch, long scratch_floats, int dtype,
+                 umb_stream_t stream);
 
 /* ---- matrix memory with exponential gates.  Per (token, head), from columns i_col / f_col of proj: i = cap tanh(z_i / cap),
  * f = log sigmoid(cap tanh(z_f / cap)).  mscan: the running maximum m_t = max(f_t + m_(t-1), i_t) of every stretch (tiles of 64 tokens

@@ -228,7 +228,7 @@ def test_retention_long_stretches_in_chunks(lib, H, D, Dv, rot, splits):
 
 
 # ------------------------------------------------------------------ convolved attention with capped scores
-def _run_conv_attention(lib, m, w, X, splits, dtype, page=4, cache=None, seq="s", raw=None):
+def _run_conv_attention(lib, m, w, X, splits, dtype, page=4, cache=None, seq="s", raw=None, split_rows=True):
     from umbrella_amd.attn.cache import PagedSeqCache
     from umbrella_amd.models.config import rotary_frequencies
     H, G, D, E, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
@@ -246,6 +246,7 @@ def _run_conv_attention(lib, m, w, X, splits, dtype, page=4, cache=None, seq="s"
     cache.open(seq)
     kv = cache.struct(0)
     conv = dev(torch.cat([w["q.conv"], w["k.conv"], w["v.conv"]]), dtype)
+    scratch2 = zeros(64 * (C + 64))                       # with it, steps of few tokens convolve over (token, 256 channels)
     outs, at = [], 0
     for cnt in splits:
         p0 = cache.extend(seq, cnt)
@@ -254,7 +255,8 @@ def _run_conv_attention(lib, m, w, X, splits, dtype, page=4, cache=None, seq="s"
         q, out = zeros(cnt, H * D), zeros(cnt, H * E + 3, dtype=dtype)
         single = int(cnt == 1)
         call("umb_cva_prep", q, kv, proj, ld, conv, cache.mixer_conv[0], dev(w["q.norm"], dtype), dev(w["k.norm"], dtype), st.d["pos"],
-             st.d["slot"], fr, cnt, H, G, D, E, taps, rot["dims"], 1, single, 1e-5, code(dtype))
+             st.d["slot"], fr, cnt, H, G, D, E, taps, rot["dims"], 1, single, 1e-5, scratch2 if split_rows else None,
+             scratch2.numel() if split_rows else 0, code(dtype))
         if not single:
             call("umb_ssd_conv_update", cache.mixer_conv[0], proj, ld, 0, st.d["seq_slot"], st.d["seq_row0"], st.d["seq_pos0"],
                  st.d["seq_len"], 1, C, taps)
@@ -287,7 +289,8 @@ def _conv_attention_case(H, G, D, E, taps, dims, scaling, softcap, seed, n, W=24
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,E,taps,dims,scaling,softcap,splits",
                          [(4, 2, 8, 6, 3, 4, True, 3.0, [19]), (3, 1, 7, 9, 1, 6, False, 50.0, [1] * 11), (2, 2, 16, 16, 4, 16, True, 2.0, [2, 2, 7, 1, 1, 16, 3]),
-                          (8, 2, 32, 48, 2, 8, True, 4.0, [30, 1, 1, 17, 2]), (4, 4, 8, 16, 5, 0, False, 8.0, [3, 2, 2, 1, 1, 1, 6])])
+                          (8, 2, 32, 48, 2, 8, True, 4.0, [30, 1, 1, 17, 2, 70, 1]), (4, 4, 8, 16, 5, 0, False, 8.0, [3, 2, 2, 1, 1, 1, 6]),
+                          (2, 1, 8, 8, 9, 4, False, 6.0, [5, 1, 1, 4, 1, 12])])
 def test_convolved_attention_prompt_portions_and_single_tokens(lib, dtype, H, G, D, E, taps, dims, scaling, softcap, splits):
     from oracle import zusuvik as O
     n = sum(splits)
@@ -296,6 +299,8 @@ def test_convolved_attention_prompt_portions_and_single_tokens(lib, dtype, H, G,
     want, _ = O.conv_attention(X.double(), torch.arange(n), m, wd, 1e-5)
     got, cache = _run_conv_attention(lib, m, {k: v.to(dtype).float() for k, v in w.items()}, X, splits, dtype)
     assert close(got, 0.8 * want, F32_TOL if dtype == torch.float32 else BF16_TOL)
+    one, _ = _run_conv_attention(lib, m, {k: v.to(dtype).float() for k, v in w.items()}, X, splits, dtype, split_rows=False)
+    assert close(one, 0.8 * want, F32_TOL if dtype == torch.float32 else BF16_TOL)       # one workgroup per token whatever the step
     # the pages and the slot go back and are used again by a sequence that starts at 0
     cache.close("s")
     again, _ = _run_conv_attention(lib, m, {k: v.to(dtype).float() for k, v in w.items()}, X[:9], [4, 1, 4], dtype, cache=cache, seq="t")

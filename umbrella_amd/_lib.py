@@ -320,7 +320,7 @@ SEQ_SIGNATURES = {
     "umb_rope_scale": [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F],
     "umb_decay_fill": [_P, _P, _P, _I, _I],
     "umb_head_gate": [_P, _I, _P, _I, _I, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _F, _I],
-    "umb_cva_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I],
+    "umb_cva_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P, _L, _I],
     "umb_mlstm_mscan": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _P, _P, _P, _I, _I],
     "umb_mlstm_prep": [_P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _F],
     "umb_mlstm_step": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _F],

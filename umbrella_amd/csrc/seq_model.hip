@@ -236,8 +236,9 @@ static int mix_attn_mlstm(const UmbSeqModel* m, const UmbSeqLayer& ly, const Umb
   const long spare2_floats = ws->aux_floats - (long)(spare2 - ws->aux);
   if (spare2_floats < 0) return UMB_EINVAL;
   const int single = s->max_len == 1;                        // one token per sequence: the ring is refreshed inside prep
+  // (what lies behind the queries is scratch until the memory's part begins: the convolved row of few-token steps, split keys)
   SEQ_TRY(umb_cva_prep(q, &ly.kv, ws->proj, ld, ly.c_conv, ly.c_conv_state, ly.q_norm, ly.k_norm, s->pos, s->slot, ly.rot_freq, T, H, G,
-                       D, E, ly.c_taps, ly.rot_dims, ly.rot_layout, single, m->eps, dt, st));
+                       D, E, ly.c_taps, ly.rot_dims, ly.rot_layout, single, m->eps, qs, ws->aux_floats - (long)(qs - ws->aux), dt, st));
   if (!single && ly.c_conv)
     SEQ_TRY(umb_ssd_conv_update(ly.c_conv_state, ws->proj, ld, 0, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B, C, ly.c_taps, st));
   if (s->max_len >= 16 && umb_bsa_attend_tiled_ok(H, G, D, E, dt))

@@ -311,8 +311,10 @@ class SeqMixLM(LLMBase):
                     mix=m.heads * m.vdim)
             elif m.kind == "attention_mlstm":
                 # aux: queries | scaled memory queries | widened values | gates, decays, logarithms, maxima | chunk states
+                # (before the memory's part begins the same room holds the convolved [q | k] row and its partial sums of few-token steps)
                 chunk = m.m_heads * (m.m_dim * m.m_pad + 1)
-                ask(aux=m.heads * m.dim + m.m_heads * (m.m_dim + m.m_pad + 5) + (chunk + 63) // 64 + (8 * chunk + 64) // T + 1,
+                conv_row = (m.heads + m.kv_heads) * m.dim + 2 * (((m.heads + m.kv_heads) * m.dim + m.kv_heads * m.vdim + 255) // 256)
+                ask(aux=m.heads * m.dim + max(conv_row, m.m_heads * (m.m_dim + m.m_pad + 5) + (chunk + 63) // 64 + (8 * chunk + 64) // T + 1),
                     o=m.m_heads * m.m_pad, mix=m.heads * m.vdim + m.m_heads * m.m_vdim)
             else:
                 ask(aux=m.heads * m.dim, o=m.heads * m.vdim, mix=m.heads * m.vdim)
