@@ -54,12 +54,12 @@ def test_synthetic_checkpoint_names_and_shapes():
     assert sd["l0.mix.g"].shape == (18, 40) and sd["l1.mix.right.i.b"].shape == (3,)
 
 
-@pytest.mark.parametrize("scaling", [None, {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048},
+@pytest.mark.parametrize("scaling", [None, {"factor": 16.0, "low": 1.0, "high": 8.0, "original": 4096},
                                      {"factor": 3.0, "low": 2.0, "high": 5.0, "original": 100}])
 def test_rotary_frequency_table_equals_the_scalar_statement(scaling):
     from oracle import zusuvik as O
     from umbrella_amd.models.config import rotary_frequencies
-    for dims, base in ((16, 500000.0), (6, 50.0), (64, 10000.0)):
+    for dims, base in ((24, 250000.0), (6, 50.0), (64, 10000.0)):
         rot = {"dims": dims, "base": base}
         if scaling:
             rot["scaling"] = scaling
