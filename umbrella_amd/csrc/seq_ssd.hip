@@ -159,14 +159,17 @@ struct ScArgs {
   const int *seq_slot, *seq_row0, *seq_pos0, *seq_len;
 };
 
-// inclusive prefix sums of the chunk's log decays into cum[SC_Q] (tokens past the stretch add nothing); one wave
-__device__ __forceinline__ void sc_cumsum(float* cum, const ScArgs& a, long row0, int cnt, int h) {
+// inclusive prefix sums of the chunk's log decays into cum[SC_Q] (tokens past the stretch add nothing); one wave.  The sums are
+// kept in double: a decay between two tokens of a chunk is the exponential of a DIFFERENCE of two prefix sums, and with strong
+// decays (logarithms of -10 and below) fp32 prefix sums of a few hundred would leave that difference good to 1e-5 only, where
+// the token-by-token recurrence multiplies by every decay itself.
+__device__ __forceinline__ void sc_cumsum(double* cum, const ScArgs& a, long row0, int cnt, int h) {
   const int lane = threadIdx.x;
   if (lane < 64) {
-    float v = lane < cnt ? a.la[(row0 + lane) * a.H + h] : 0.f;
+    double v = lane < cnt ? (double)a.la[(row0 + lane) * a.H + h] : 0.0;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
-      const float u = __shfl_up(v, o, 64);
+      const double u = __shfl_up(v, o, 64);
       if (lane >= o) v += u;
     }
     cum[lane] = v;
@@ -181,16 +184,16 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(float* __restrict_
   if (t0 >= len) return;
   const int cnt = len - t0 < SC_Q ? len - t0 : SC_Q, N = a.N, P = a.P;
   const long row0 = a.seq_row0[b] + t0;
-  float* cum = sm;                         // [64]
-  float* kw = sm + 64;                     // [Q][N]: k_s * exp(c_Q - c_s)
+  double* cum = reinterpret_cast<double*>(sm);   // [64] doubles
+  float* kw = sm + 128;                    // [Q][N]: k_s * exp(c_Q - c_s)
   float* vs = kw + SC_Q * N;               // [Q][16]
   sc_cumsum(cum, a, row0, cnt, h);
   __syncthreads();
-  const float cend = cum[SC_Q - 1];
+  const double cend = cum[SC_Q - 1];
   const int g = h / a.hpg;
   for (int i = threadIdx.x; i < SC_Q * N; i += 256) {
     const int s = i / N, n = i % N;
-    kw[i] = s < cnt ? a.k[(row0 + s) * a.ldk + (long)g * N + n] * expf(cend - cum[s]) : 0.f;
+    kw[i] = s < cnt ? a.k[(row0 + s) * a.ldk + (long)g * N + n] * expf((float)(cend - cum[s])) : 0.f;
   }
   for (int i = threadIdx.x; i < SC_Q * 16; i += 256) {
     const int s = i >> 4, p = p0 + (i & 15);
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(float* __restrict_
     for (int j = 0; j < 16; ++j)
       if (p0 + j < P) dst[j] = acc[j];
   }
-  if (threadIdx.x == 0 && blockIdx.x == 0) ac[((long)b * a.H + h) * a.max_chunks + c] = expf(cend);
+  if (threadIdx.x == 0 && blockIdx.x == 0) ac[((long)b * a.H + h) * a.max_chunks + c] = expf((float)cend);
 }
 
 // (2) start states: thread per state element of a (sequence, head), chunks in order; sc[c] becomes the START state of chunk c
@@ -242,8 +245,8 @@ __global__ __launch_bounds__(256) void ssd_chunk_out_kernel(float* __restrict__ 
   if (t0 >= len) return;
   const int cnt = len - t0 < SC_Q ? len - t0 : SC_Q, N = a.N, P = a.P, NL = N + 1;
   const long row0 = a.seq_row0[b] + t0;
-  float* cum = sm;                         // [64]
-  float* qs = sm + 64;                     // [Q][N + 1]
+  double* cum = reinterpret_cast<double*>(sm);   // [64] doubles
+  float* qs = sm + 128;                    // [Q][N + 1]
   float* kt = qs + SC_Q * NL;              // [N][Q] keys transposed; later the start state [N][SC_PS]
   float* vs = kt + (N * SC_Q > N * SC_PS ? N * SC_Q : N * SC_PS);   // [Q][SC_PS]
   float* ms = vs + SC_Q * SC_PS;           // [Q][Q + 1]: decayed, masked scores
@@ -275,11 +278,11 @@ __global__ __launch_bounds__(256) void ssd_chunk_out_kernel(float* __restrict__ 
       for (int e = 0; e < 4; ++e) acc[4 * j4 + e] += qv * kk[e];
     }
   }
-  const float ct = cum[t];
+  const double ct = cum[t];
 #pragma unroll
   for (int j = 0; j < 16; ++j) {
     const int s = 16 * qd + j;
-    ms[t * (SC_Q + 1) + s] = s <= t ? acc[j] * expf(ct - cum[s]) : 0.f;
+    ms[t * (SC_Q + 1) + s] = s <= t ? acc[j] * expf((float)(ct - cum[s])) : 0.f;
   }
   __syncthreads();                          // scores are in ms, kt is free: bring in the chunk's start state
   const float* s0 = sc + ((((long)b * a.H + h) * a.max_chunks + c) * N) * P;
@@ -312,7 +315,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_out_kernel(float* __restrict__ 
     }
   }
   if (t < cnt) {
-    const float et = expf(ct);
+    const float et = expf((float)ct);
     float* dst = o + (row0 + t) * ((long)a.H * P) + (long)h * P + p0 + 16 * qd;
 #pragma unroll
     for (int j = 0; j < 16; ++j)
@@ -322,7 +325,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_out_kernel(float* __restrict__ 
 
 static inline size_t sc_out_lds(int N) {
   const size_t kt = (size_t)N * (SC_Q > SC_PS ? SC_Q : SC_PS);
-  return (64 + (size_t)SC_Q * (N + 1) + kt + (size_t)SC_Q * SC_PS + (size_t)SC_Q * (SC_Q + 1)) * sizeof(float);
+  return (128 + (size_t)SC_Q * (N + 1) + kt + (size_t)SC_Q * SC_PS + (size_t)SC_Q * (SC_Q + 1)) * sizeof(float);
 }
 
 // floats of scratch the chunked form needs for a step of B stretches, the longest max_len tokens; 0: the shape is not covered
@@ -345,7 +348,7 @@ extern "C" int umb_ssd_scan_chunked(float* o, float* state, const float* q, int 
   ScArgs a{q, k, v, log_alpha, ldq, ldk, ldv, H, H / qk_heads, N, P, chunks, seq_slot, seq_row0, seq_pos0, seq_len};
   float* sc = scratch;
   float* ac = scratch + (long)B * H * chunks * N * P;
-  const size_t lds1 = (64 + (size_t)SC_Q * N + SC_Q * 16) * sizeof(float), lds3 = sc_out_lds(N);
+  const size_t lds1 = (128 + (size_t)SC_Q * N + SC_Q * 16) * sizeof(float), lds3 = sc_out_lds(N);
   if (ensure_dynamic_lds<ssd_chunk_state_kernel>(lds1) != UMB_OK || ensure_dynamic_lds<ssd_chunk_out_kernel>(lds3) != UMB_OK)
     return UMB_EHIP;
   hipLaunchKernelGGL(ssd_chunk_state_kernel, dim3((P + 15) / 16, chunks, B * H), dim3(256), lds1, st, sc, ac, a);
